@@ -1,0 +1,625 @@
+// FP8 (OCP e4m3fn) skinny GEMM for MI355X / gfx950:  D[m,n] (+)= sa[m] * sb[n] * sum_k A[m,k] * W[n,k],  m <= 64.
+//
+// Replaces the reference's persistent producer/consumer kernel and its consumers
+// (csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79, producers/n_full_tiles.cu:4-127,
+// consumers/mfma_16x16x32_consumer.cu:1-168, consumers/smfma_16x16x64_consumer.cu:1-158) with a different
+// design: the op is a pure weight stream (2*m flop per weight byte against ~625 flop/byte of machine balance),
+// so everything is organised around keeping 16-byte, fully coalesced, non-temporal weight loads in flight.
+//
+//  * Work unit = (panel of 16*WN weight rows) x (K slab of 256*WK*CH bytes).  Units are ordered slab-fastest and
+//    cut into `grid` equal contiguous ranges, one per persistent workgroup (stream-K): every CU streams the same
+//    number of bytes whatever the shape.  Logical workgroup ids are laid out so that one XCD owns one contiguous
+//    range of units (neighbouring workgroups, which may share a panel, share an L2).
+//  * A workgroup is 8 waves = WN (rows) x WK (K).  Per 256-byte K chunk a wave issues four 16-byte buffer loads
+//    per lane, each instruction covering 4 weight rows x 256 contiguous bytes (two full cache lines per row),
+//    `nt` so the stream does not displace the activations in L2.  Two units are always in flight per wave.
+//  * The chunk is turned into MFMA operand layout (lane = row + 16*kgroup, 32 contiguous K bytes per lane)
+//    through a wave-private, XOR-swizzled 4 KB LDS tile: no barrier, the wave only waits on its own LDS ops.
+//  * The activation slab [16*MT, KS] is staged in LDS once per unit for all 8 waves (double buffered, same
+//    swizzle), so the only global traffic in the loop is the weight stream.
+//  * Contraction: v_mfma_f32_16x16x128_f8f6f4, weights as the A operand (rows = n), activations as the
+//    B operand (cols = m), fp32 accumulators held across all the slabs a workgroup owns of a panel.
+//  * When a panel ends: waves that split K inside the workgroup are summed through LDS; if the workgroup owned
+//    every slab of the panel it writes D directly, otherwise it parks its fp32 partial in the workspace and the
+//    workgroup that arrives last (per-panel counter) adds the partials in workgroup order -- a fixed order, so
+//    results are bit-reproducible -- applies the scales once, adds D (accumulate mode) and rounds once.
+#include <mutex>
+#include <type_traits>
+
+#include "hfrk_internal.h"
+
+namespace hfrk {
+
+constexpr int kGemmWaves = 8;
+constexpr int kGemmThreads = kGemmWaves * kWave;
+constexpr int kTileBytes = 4096;                 // 16 rows x 256 B, one chunk of one wave
+constexpr int kLdsLimit = 160 * 1024;            // LDS per CU on gfx950
+constexpr int kMaxPanels = 1 << 20;              // per-panel arrival counters
+constexpr size_t kWsFloats = (size_t)2 * kNumCU * kGemmWaves * 4 * 256;  // 2 slots x grid x WN*MT KB (worst case)
+
+struct GemmArgs {
+    const uint8_t* A;
+    const uint8_t* B;
+    void* D;
+    const float* scale_a;
+    const float* scale_b;
+    int sa_stride, sb_stride;
+    int m, n, k, b_stride;
+    int d_dtype, accumulate;
+    int panels, slabs, units, grid, nbuf;
+    float* ws;
+    int* counters;
+};
+
+// first unit of logical workgroup g
+__device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (int)(((long)g * units) / grid); }
+
+template <int MT, int WN, int WK, int CH>
+__global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArgs a) {
+    static_assert(WN * WK == kGemmWaves, "a workgroup is 8 waves");
+    constexpr int KS = 256 * WK * CH;        // bytes of K per slab
+    constexpr int BN = 16 * WN;              // weight rows per panel
+    constexpr int ACT_BYTES = 16 * MT * KS;  // one staged activation slab
+    constexpr int KP = KS / 16;              // 16-byte pieces per activation row of a slab
+    constexpr int PIECES = 16 * MT * KP;
+    constexpr int APT = (PIECES + kGemmThreads - 1) / kGemmThreads;  // activation pieces per thread
+
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t* const tbuf_all = lds;
+    uint8_t* const act_all = lds + kGemmWaves * kTileBytes;
+    int* const flag = reinterpret_cast<int*>(act_all + 2 * ACT_BYTES);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave / WK, wk = wave % WK;
+    const int li = lane & 15, lg = lane >> 4;
+
+    const int G = a.grid, S = a.slabs, U = a.units;
+    const int b = blockIdx.x;
+    const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;  // XCD x owns logical ids [x*G/8, (x+1)*G/8)
+    const int u0 = unit_begin(g, U, G), u1 = unit_begin(g + 1, U, G);
+    if (u0 >= u1) return;  // cannot happen when grid <= units; uniform for the whole workgroup
+
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
+    uint16_t* const D = reinterpret_cast<uint16_t*>(a.D);
+
+    // ---- per-panel epilogue inputs, fetched when the panel's first weight loads are issued -------------------
+    // The vector-memory counter retires in issue order, so a load issued at the end of a panel would wait for
+    // every prefetched weight chunk; issued up front, D and the channel scales are long home when needed.
+    // A lane owns D[mt*16 + li][n0 .. n0+3], n0 = panel*BN + wn*16 + 4*lg.  At most two panels are open at once.
+    uint2 dq[2][MT];
+    float sbq[2][4];
+    float saq[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int mrow = min(mt * 16 + li, a.m - 1);
+        saq[mt] = a.scale_a[(long)mrow * a.sa_stride];
+    }
+    const bool n_vec = (a.n & 3) == 0;
+    auto panel_fetch = [&](int panel, uint2 (&dd)[MT], float (&sb)[4]) {
+        const int n0 = panel * BN + wn * 16 + 4 * lg;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int n = min(n0 + v, a.n - 1);
+            sb[v] = a.scale_b ? a.scale_b[(long)n * a.sb_stride] : 1.0f;
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            dd[mt] = make_uint2(0u, 0u);
+            const int mrow = mt * 16 + li;
+            if (a.accumulate && mrow < a.m) {
+                const uint16_t* const drow = D + (long)mrow * a.n;
+                if (n_vec && n0 + 3 < a.n) {
+                    dd[mt] = *reinterpret_cast<const uint2*>(drow + n0);
+                } else {
+                    uint32_t e[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) e[v] = (n0 + v < a.n) ? drow[n0 + v] : 0u;
+                    dd[mt] = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+                }
+            }
+        }
+    };
+    int fetch_par = 0;  // which of the two contexts the next panel_fetch fills
+
+    // ---- weight stream -------------------------------------------------------------------------------------
+    // load t of a chunk: lane -> weight row 4t + lane/16, bytes (lane%16)*16 .. +16 of the 256-byte chunk
+    const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
+    v4i wq[2][CH][4];
+    int ip = u0 / S, is = u0 % S;  // (panel, slab) of the next unit to issue
+    bool issue_first = true;       // next unit to issue opens a panel for this workgroup
+    // Every step issues the same number of loads, in range or not: a unit past the end of this workgroup's range
+    // is requested at an offset beyond the buffer, which returns zeros without touching memory.  That keeps the
+    // count of loads in flight a compile-time constant, so each wait leaves exactly the prefetched unit pending.
+    auto issue_unit = [&](auto sel, bool in_range) {
+        constexpr int X = decltype(sel)::value;
+        if (in_range && issue_first) {
+            if (wk == 0) {
+                if (fetch_par) panel_fetch(ip, dq[1], sbq[1]);
+                else panel_fetch(ip, dq[0], sbq[0]);
+            }
+            fetch_par ^= 1;
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)is * KS +
+                                                 (uint32_t)(c * WK + wk) * 256u
+                                           : 0x80000000u;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(
+                    w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+        }
+        issue_first = false;
+        if (++is == S) { is = 0; ++ip; issue_first = true; }
+    };
+
+    // ---- activation slab staging ---------------------------------------------------------------------------
+    v4i aq[APT];
+    auto act_load = [&](int slab, bool in_range) {
+        const uint32_t base = in_range ? (uint32_t)slab * KS : 0x80000000u;
+#pragma unroll
+        for (int q = 0; q < APT; ++q) {
+            const int idx = tid + q * kGemmThreads;
+            if (PIECES % kGemmThreads == 0 || idx < PIECES) {
+                const int row = idx / KP, kp = idx % KP;
+                aq[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    a_rsrc, (int)((uint32_t)row * (uint32_t)a.k + base + (uint32_t)kp * 16u), 0, 0);
+            }
+        }
+    };
+    auto act_store = [&](int buf) {
+        uint8_t* const dst = act_all + buf * ACT_BYTES;
+#pragma unroll
+        for (int q = 0; q < APT; ++q) {
+            const int idx = tid + q * kGemmThreads;
+            if (PIECES % kGemmThreads == 0 || idx < PIECES) {
+                const int row = idx / KP, kp = idx % KP;
+                *reinterpret_cast<v4i*>(dst + row * KS + (kp >> 4) * 256 + (((kp & 15) ^ (row & 15)) << 4)) = aq[q];
+            }
+        }
+    };
+
+    v4f acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    uint8_t* const tb = tbuf_all + wave * kTileBytes;
+    // swizzled offsets of this lane inside a 16 x 256 B tile: as writer (row 4t+lg, piece li) and as reader (row li)
+    int wr_off[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int row = 4 * t + lg;
+        wr_off[t] = row * 256 + ((li ^ row) << 4);
+    }
+    int rd_off[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) rd_off[h] = ((((8 * h + 2 * lg) ^ li) & 15) << 4);  // piece 8h+2g; its pair is ^16
+
+    auto consume_unit = [&](auto sel, int buf) {
+        constexpr int X = decltype(sel)::value;
+        const uint8_t* const act = act_all + buf * ACT_BYTES;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tb + wr_off[t]) = wq[X][c][t];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int kblk = c * WK + wk;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const v4i wlo = *reinterpret_cast<const v4i*>(tb + li * 256 + rd_off[h]);
+                const v4i whi = *reinterpret_cast<const v4i*>(tb + li * 256 + (rd_off[h] ^ 16));
+                const v8i wop = {wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const uint8_t* const arow = act + (mt * 16 + li) * KS + kblk * 256;
+                    const v4i alo = *reinterpret_cast<const v4i*>(arow + rd_off[h]);
+                    const v4i ahi = *reinterpret_cast<const v4i*>(arow + (rd_off[h] ^ 16));
+                    const v8i aop = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+                    acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc[mt], 0, 0, 0, 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
+
+    // ---- epilogue ------------------------------------------------------------------------------------------
+    // lane holds, per m-tile, D^T[n0 + v][mt*16 + li], v = 0..3: scale, add the fetched D, round once, store
+    auto store_panel = [&](int panel, int par) {
+        const int n0 = panel * BN + wn * 16 + 4 * lg;
+        const bool vec_ok = n_vec && (n0 + 3 < a.n);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int mrow = mt * 16 + li;
+            if (mrow >= a.m) continue;
+            const uint2 old = par ? dq[1][mt] : dq[0][mt];
+            const uint32_t oe[4] = {old.x & 0xffffu, old.x >> 16, old.y & 0xffffu, old.y >> 16};
+            uint32_t o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float r = acc[mt][v] * (saq[mt] * (par ? sbq[1][v] : sbq[0][v]));
+                if (a.d_dtype == HFRK_BF16) o[v] = store16<HFRK_BF16>(a.accumulate ? load16<HFRK_BF16>((uint16_t)oe[v]) + r : r);
+                else o[v] = store16<HFRK_F16>(a.accumulate ? load16<HFRK_F16>((uint16_t)oe[v]) + r : r);
+            }
+            uint16_t* const drow = D + (long)mrow * a.n;
+            if (vec_ok) {
+                *reinterpret_cast<uint2*>(drow + n0) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n0 + v < a.n) drow[n0 + v] = (uint16_t)o[v];
+            }
+        }
+    };
+
+    // fp32 partial of (workgroup gg, slot): [wn][mt][lane] float4
+    auto ws_ptr = [&](int gg, int slot) -> v4f* {
+        return reinterpret_cast<v4f*>(a.ws) + ((size_t)(gg * 2 + slot) * (WN * MT)) * 64;
+    };
+
+    int flush_par = 0;  // context of the panel that closes next
+    // close panel `panel`, of which this workgroup covered slabs [s_first, s_end)
+    auto flush_panel = [&](int panel, int s_first, int s_end) {
+        if constexpr (WK > 1) {
+            // sum the WK waves that share rows; their transposition tiles are idle here and serve as scratch
+            v4f* const mine = reinterpret_cast<v4f*>(tb);
+            if (wk != 0) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) mine[mt * 64 + lane] = acc[mt];
+            }
+            __syncthreads();
+            if (wk == 0) {
+#pragma unroll
+                for (int w = 1; w < WK; ++w) {
+                    const v4f* const other = reinterpret_cast<const v4f*>(tbuf_all + (wn * WK + w) * kTileBytes);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[mt] += other[mt * 64 + lane];
+                }
+            }
+            __syncthreads();
+        }
+        const bool full = (s_first == 0) && (s_end == S);
+        if (full) {
+            if (wk == 0) store_panel(panel, flush_par);
+        } else {
+            const int slot = (panel == u0 / S) ? 0 : 1;
+            if (wk == 0) {
+                v4f* const dst = ws_ptr(g, slot) + (wn * MT) * 64;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) dst[mt * 64 + lane] = acc[mt];
+                __threadfence();
+            }
+            __syncthreads();
+            if (tid == 0) {
+                const int mine = s_end - s_first;
+                const int seen = atomicAdd(&a.counters[panel], mine);
+                const int last = (seen + mine == S);
+                if (last) a.counters[panel] = 0;  // ready for the next launch
+                *flag = last;
+            }
+            __syncthreads();
+            const int last = *flag;
+            if (last && wk == 0) {
+                __threadfence();
+                // contributors are the workgroups whose unit range meets [panel*S, (panel+1)*S), in id order
+                const long lo = (long)panel * S, hi = lo + S;
+                const int g_first = (int)(((lo + 1) * G + U - 1) / U) - 1;
+                const int g_last = (int)((hi * G + U - 1) / U) - 1;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+                for (int gg = g_first; gg <= g_last; ++gg) {
+                    const int sl = (unit_begin(gg, U, G) / S == panel) ? 0 : 1;
+                    const v4f* const src = ws_ptr(gg, sl) + (wn * MT) * 64;
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[mt] += __builtin_nontemporal_load(src + mt * 64 + lane);
+                }
+                store_panel(panel, flush_par);
+            }
+            __syncthreads();  // `flag` may be rewritten by the next flush
+        }
+        flush_par ^= 1;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+    };
+
+    // ---- main loop -----------------------------------------------------------------------------------------
+    // Issue order matters because loads retire in order: the activation slab of unit u+2 is requested before the
+    // weights of unit u+2, so storing it to LDS at the top of step u+1 never waits on weights still in flight.
+    using Sel0 = std::integral_constant<int, 0>;
+    using Sel1 = std::integral_constant<int, 1>;
+    int cp = u0 / S, cs = u0 % S;  // (panel, slab) of the unit being consumed
+    int s_first = cs;              // first slab this workgroup covers of the current panel
+    auto next_slab = [&](int s) { return (s + 1 == S) ? 0 : s + 1; };
+
+    act_load(cs, true);
+    issue_unit(Sel0{}, true);
+    act_store(0);
+    act_load(next_slab(cs), u0 + 1 < u1);
+    issue_unit(Sel1{}, u0 + 1 < u1);
+    __syncthreads();
+
+    // One step = one unit.  A step whose unit lies past u1 (odd range length) multiplies zeros and changes nothing.
+    auto step = [&](auto sel, int u) {
+        constexpr int X = decltype(sel)::value;
+        const int ns = next_slab(cs);
+        if (u + 1 < u1) act_store(X ^ 1);  // slab of unit u+1, requested one step ago
+        consume_unit(sel, X);
+        if (u < u1 && (u + 1 == u1 || ns == 0)) {
+            flush_panel(cp, s_first, cs + 1);
+            s_first = 0;
+        }
+        act_load(next_slab(ns), u + 2 < u1);
+        issue_unit(sel, u + 2 < u1);
+        if (u + 1 < u1) __syncthreads();
+        cs = ns;
+        if (ns == 0) ++cp;
+    };
+    for (int u = u0; u < u1; u += 2) {
+        step(Sel0{}, u);
+        step(Sel1{}, u + 1);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------------------
+struct DeviceState {
+    float* ws = nullptr;
+    int* counters = nullptr;
+};
+static DeviceState g_dev[64];
+static std::mutex g_mutex;
+
+static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
+    if (dev < 0 || dev >= 64) return HFRK_BAD_SHAPE;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if (g_dev[dev].ws != nullptr) {
+            *out = &g_dev[dev];
+            return HFRK_SUCCESS;
+        }
+    }
+    if (stream != nullptr) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+            return HFRK_NOT_INITIALISED;
+    }
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_dev[dev].ws == nullptr) {
+        float* ws = nullptr;
+        int* counters = nullptr;
+        HFRK_HIP_TRY(hipMalloc(&ws, kWsFloats * sizeof(float)));
+        hipError_t e = hipMalloc(&counters, kMaxPanels * sizeof(int));
+        if (e == hipSuccess) e = hipMemset(counters, 0, kMaxPanels * sizeof(int));
+        if (e != hipSuccess) {
+            (void)hipFree(ws);
+            if (counters) (void)hipFree(counters);
+            set_last_hip_error(e);
+            return HFRK_HIP_ERROR;
+        }
+        g_dev[dev].counters = counters;
+        g_dev[dev].ws = ws;
+    }
+    *out = &g_dev[dev];
+    return HFRK_SUCCESS;
+}
+
+static int lds_bytes_for(int mt, int wk, int ch) {
+    const int ks = 256 * wk * ch;
+    return kGemmWaves * kTileBytes + 2 * 16 * mt * ks + 16;
+}
+
+// Rough time model of one candidate decomposition, in nanoseconds; only its ordering matters.
+static double plan_cost(int n, int k, int mt, int wn, int wk, int ch, int* grid_out) {
+    const int bn = 16 * wn, ks = 256 * wk * ch;
+    const int panels = (n + bn - 1) / bn, slabs = k / ks;
+    const long units = (long)panels * slabs;
+    const int grid = (int)(units < kNumCU ? units : kNumCU);
+    *grid_out = grid;
+    const long upw = (units + grid - 1) / grid;                    // units of the busiest workgroup
+    const double cu_bw = 27.0;                                     // bytes/ns one CU sustains (~6.9 TB/s / 256)
+    const double stream = (double)upw * bn * ks / cu_bw;           // streaming time
+    const double per_unit = 120.0;                                 // barrier + slab staging exposure
+    const double panels_per_wg = (double)upw / slabs + 1.0;
+    const double flush = (wk > 1 ? 250.0 : 80.0) * panels_per_wg;  // in-workgroup reduction + store
+    const bool aligned = (units % grid == 0) && ((units / grid) % slabs == 0);
+    const double fixup = aligned ? 0.0 : 1500.0;                   // workspace round trip of shared panels
+    const double waste = (double)(panels * bn - n) / n;            // rows streamed past n cost no traffic but idle waves
+    return (stream + upw * per_unit + flush + fixup) * (1.0 + waste);
+}
+
+static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
+    if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    const int mt = (m + 15) / 16;
+    static const int wns[4] = {1, 2, 4, 8};
+    double best = 1e300;
+    bool found = false;
+    for (int wi = 0; wi < 4; ++wi) {
+        for (int ch = 2; ch >= 1; --ch) {
+            const int wn = wns[wi], wk = kGemmWaves / wn;
+            const int ks = 256 * wk * ch;
+            if (k % ks != 0) continue;
+            if (lds_bytes_for(mt, wk, ch) > kLdsLimit) continue;
+            const int bn = 16 * wn;
+            const long panels = (n + bn - 1) / bn;
+            if (panels > kMaxPanels) continue;
+            int grid;
+            const double c = plan_cost(n, k, mt, wn, wk, ch, &grid);
+            if (c < best) {
+                best = c;
+                found = true;
+                plan->m_tiles = mt;
+                plan->wn = wn;
+                plan->wk = wk;
+                plan->ch = ch;
+                plan->grid = grid;
+                plan->panels = (int)panels;
+                plan->slabs = k / ks;
+                plan->lds_bytes = lds_bytes_for(mt, wk, ch);
+            }
+        }
+    }
+    return found ? HFRK_SUCCESS : HFRK_BAD_SHAPE;
+}
+
+static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
+    if (p->m_tiles < 1 || p->m_tiles > 4 || p->m_tiles * 16 < m) return HFRK_INVALID_CONFIG;
+    if (!(p->wn == 1 || p->wn == 2 || p->wn == 4 || p->wn == 8) || p->wn * p->wk != kGemmWaves) return HFRK_INVALID_CONFIG;
+    if (p->ch != 1 && p->ch != 2) return HFRK_INVALID_CONFIG;
+    const int ks = 256 * p->wk * p->ch, bn = 16 * p->wn;
+    if (k % ks != 0 || p->slabs != k / ks || p->panels != (n + bn - 1) / bn) return HFRK_INVALID_CONFIG;
+    if (p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
+    const long units = (long)p->panels * p->slabs;
+    if (p->grid < 1 || p->grid > kNumCU || p->grid > units) return HFRK_INVALID_CONFIG;
+    if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
+    return HFRK_SUCCESS;
+}
+
+template <int MT, int WN, int WK, int CH>
+static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    auto kern = skinny_gemm_kernel<MT, WN, WK, CH>;
+    static bool attr_done[64] = {};
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    if (dev >= 0 && dev < 64 && !attr_done[dev]) {
+        HFRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        attr_done[dev] = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}
+
+template <int MT>
+static int launch_mt(const GemmArgs& args, const hfrk_gemm_plan& p, hipStream_t stream) {
+#define HFRK_CASE(WN_, WK_, CH_) \
+    if (p.wn == WN_ && p.ch == CH_) return launch_one<MT, WN_, WK_, CH_>(args, p.lds_bytes, stream);
+    HFRK_CASE(1, 8, 1) HFRK_CASE(1, 8, 2) HFRK_CASE(2, 4, 1) HFRK_CASE(2, 4, 2)
+    HFRK_CASE(4, 2, 1) HFRK_CASE(4, 2, 2) HFRK_CASE(8, 1, 1) HFRK_CASE(8, 1, 2)
+#undef HFRK_CASE
+    return HFRK_INVALID_CONFIG;
+}
+
+static int gemm_launch(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
+                       const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
+                       int accumulate, const hfrk_gemm_plan* user_plan, hipStream_t stream) {
+    if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
+    if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (d_dtype != HFRK_F16 && d_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
+    if (!A || !B || !D || !scale_a) return HFRK_BAD_SHAPE;
+    if ((sa_stride != 0 && sa_stride != 1) || (sb_stride != 0 && sb_stride != 1)) return HFRK_BAD_SHAPE;
+    // every offset the kernel forms, including rows of the last (padded) panel, must stay below 2^31
+    if (((long)n + 128) * b_stride + k >= (1L << 31) || (long)m * k >= (1L << 31)) return HFRK_BAD_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15 || (b_stride & 15)) return HFRK_BAD_ALIGNMENT;
+    if (reinterpret_cast<uintptr_t>(D) & 1) return HFRK_BAD_ALIGNMENT;
+
+    hfrk_gemm_plan p;
+    if (user_plan) {
+        p = *user_plan;
+        const int rc = check_plan(m, n, k, &p);
+        if (rc != HFRK_SUCCESS) return rc;
+    } else {
+        const int rc = make_plan(m, n, k, &p);
+        if (rc != HFRK_SUCCESS) return rc;
+    }
+
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    DeviceState* st = nullptr;
+    const int rc = ensure_workspace(dev, stream, &st);
+    if (rc != HFRK_SUCCESS) return rc;
+
+    GemmArgs args;
+    args.A = static_cast<const uint8_t*>(A);
+    args.B = static_cast<const uint8_t*>(B);
+    args.D = D;
+    args.scale_a = scale_a;
+    args.scale_b = scale_b;
+    args.sa_stride = sa_stride;
+    args.sb_stride = sb_stride;
+    args.m = m;
+    args.n = n;
+    args.k = k;
+    args.b_stride = b_stride;
+    args.d_dtype = d_dtype;
+    args.accumulate = accumulate;
+    args.panels = p.panels;
+    args.slabs = p.slabs;
+    args.units = p.panels * p.slabs;
+    args.grid = p.grid;
+    args.nbuf = 2;
+    args.ws = st->ws;
+    args.counters = st->counters;
+    // the vector store path needs 8-byte aligned rows
+    if ((reinterpret_cast<uintptr_t>(D) & 7) != 0 && (n & 3) == 0) {
+        // D rows would be misaligned for 8-byte stores: report rather than take a slow path silently
+        return HFRK_BAD_ALIGNMENT;
+    }
+    switch (p.m_tiles) {
+        case 1: return launch_mt<1>(args, p, stream);
+        case 2: return launch_mt<2>(args, p, stream);
+        case 3: return launch_mt<3>(args, p, stream);
+        case 4: return launch_mt<4>(args, p, stream);
+    }
+    return HFRK_INVALID_CONFIG;
+}
+
+}  // namespace hfrk
+
+extern "C" {
+
+int hfrk_init(void) {
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    hfrk::DeviceState* st = nullptr;
+    return hfrk::ensure_workspace(dev, nullptr, &st);
+}
+
+int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, int A_producers, int B_producers,
+                              int consumers, int a_lanes, int b_lanes, int qsize, int op_m, int ops) {
+    (void)split_k;
+    // the reference derives its K tile from the MFMA shape it would use: (512/op_m) * ops
+    if (op_m != 8 && op_m != 16 && op_m != 32) return HFRK_INVALID_CONFIG;
+    const int warptile_k = (512 / op_m) * ops;
+    if (n % 2 != 0) return HFRK_N_NOT_EVEN;
+    if (warptile_k <= 0 || k % warptile_k != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (A_producers + B_producers + consumers > 16) return HFRK_TOO_MANY_WARPS;
+    if (a_lanes <= 0 || b_lanes <= 0) return HFRK_INVALID_CONFIG;
+    if (qsize < A_producers / a_lanes || qsize < B_producers / b_lanes || qsize < consumers) return HFRK_QSIZE_TOO_SMALL;
+    if (a_lanes > 4 || b_lanes > 6 || qsize < 1 || qsize > 6 || (ops != 4 && ops != 8)) return HFRK_INVALID_CONFIG;
+    // limits of this implementation
+    if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
+    if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (b_stride % 16 != 0) return HFRK_BAD_ALIGNMENT;
+    return HFRK_SUCCESS;
+}
+
+int hfrk_skinny_gemm_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (!plan) return HFRK_BAD_SHAPE;
+    return hfrk::make_plan(m, n, k, plan);
+}
+
+int hfrk_skinny_gemm(const void* A, const void* B, void* D, const float* scale_tensor, int m, int n, int k,
+                     int b_stride, int split_k, int A_producers, int B_producers, int consumers, int a_lanes,
+                     int b_lanes, int qsize, int op_m, int ops, int d_dtype, void* stream) {
+    const int rc = hfrk_skinny_gemm_validate(m, n, k, b_stride, split_k, A_producers, B_producers, consumers, a_lanes,
+                                             b_lanes, qsize, op_m, ops);
+    if (rc != HFRK_SUCCESS) return rc;
+    return hfrk::gemm_launch(A, B, D, scale_tensor, 0, nullptr, 0, m, n, k, b_stride, d_dtype, 1, nullptr,
+                             static_cast<hipStream_t>(stream));
+}
+
+int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
+                        const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
+                        int accumulate, const hfrk_gemm_plan* plan, void* stream) {
+    return hfrk::gemm_launch(A, B, D, scale_a, sa_stride, scale_b, sb_stride, m, n, k, b_stride, d_dtype, accumulate,
+                             plan, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

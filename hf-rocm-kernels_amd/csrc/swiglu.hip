@@ -1,0 +1,115 @@
+// output[r,c] = e4m3fn( clamp( silu(gate_up[r,c]) * gate_up[r,cols+c] / scale, +-448 ) );  next_buffer <- 0
+//
+// Replaces csrc/op_src/swiglu/swiglu_dispatch.cu:8-42 and its kernels (swiglu_scalar.cu:24-66,
+// swiglu_vectorized.cu:27-97).  Pure streaming op: 16-byte loads of 8 gate and 8 up values, fp32 math
+// (x * 1/(1 + 2^(-x*log2 e)), the same exp2 form as the reference), one 8-byte store of 8 fp8 values.
+// The clamp is +-448, the largest e4m3fn value (the reference's vectorised kernel clamps at 224 because its
+// fnuz encoding tops out at 240, csrc/utils/macros.h:15).
+#include "hfrk_internal.h"
+
+namespace hfrk {
+
+__device__ __forceinline__ float silu_mul(float g, float u, float inv_scale) {
+    const float e = __builtin_amdgcn_exp2f(-g * 1.44269504089f);
+    return g * __builtin_amdgcn_rcpf(1.0f + e) * u * inv_scale;
+}
+
+// Zero rows*buffer_cols 16-bit elements, spread over every thread of the grid.
+__device__ __forceinline__ void zero_next_buffer(uint16_t* next_buffer, long total) {
+    if (total <= 0) return;
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long nthreads = (long)gridDim.x * blockDim.x;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(next_buffer);
+    long head = (long)(((16 - (addr & 15)) & 15) >> 1);
+    if (head > total) head = total;
+    const long body = (total - head) >> 3;
+    for (long i = tid; i < head; i += nthreads) next_buffer[i] = 0;
+    uint4* const vec = reinterpret_cast<uint4*>(next_buffer + head);
+    for (long i = tid; i < body; i += nthreads) vec[i] = make_uint4(0, 0, 0, 0);
+    for (long i = head + body * 8 + tid; i < total; i += nthreads) next_buffer[i] = 0;
+}
+
+template <int DT>
+__global__ void __launch_bounds__(1024) swiglu_vec_kernel(const uint16_t* __restrict__ gate_up,
+                                                          const float* __restrict__ scale_tensor,
+                                                          uint8_t* __restrict__ output, uint16_t* __restrict__ next_buffer,
+                                                          int rows, int cols, int buffer_cols) {
+    const int vpr = cols >> 3;  // 8-element pieces per output row
+    const long nvec = (long)rows * vpr;
+    const float s = scale_tensor[0];
+    const float inv_scale = (s != 0.f) ? 1.f / s : 1.f;
+    for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += (long)gridDim.x * blockDim.x) {
+        const long r = v / vpr;
+        const int c = (int)(v - r * vpr);
+        const uint16_t* const grow = gate_up + r * 2 * cols;
+        const v4i g = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(grow) + c);
+        const v4i u = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(grow + cols) + c);
+        const uint32_t gw[4] = {(uint32_t)g[0], (uint32_t)g[1], (uint32_t)g[2], (uint32_t)g[3]};
+        const uint32_t uw[4] = {(uint32_t)u[0], (uint32_t)u[1], (uint32_t)u[2], (uint32_t)u[3]};
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            y[2 * j] = silu_mul(load16<DT>((uint16_t)(gw[j] & 0xffff)), load16<DT>((uint16_t)(uw[j] & 0xffff)), inv_scale);
+            y[2 * j + 1] = silu_mul(load16<DT>((uint16_t)(gw[j] >> 16)), load16<DT>((uint16_t)(uw[j] >> 16)), inv_scale);
+        }
+        uint32_t p0 = cvt_pk_fp8(y[0], y[1], 0u, false);
+        p0 = cvt_pk_fp8(y[2], y[3], p0, true);
+        uint32_t p1 = cvt_pk_fp8(y[4], y[5], 0u, false);
+        p1 = cvt_pk_fp8(y[6], y[7], p1, true);
+        reinterpret_cast<uint2*>(output + r * cols)[c] = make_uint2(p0, p1);
+    }
+    zero_next_buffer(next_buffer, (long)rows * buffer_cols);
+}
+
+template <int DT>
+__global__ void __launch_bounds__(1024) swiglu_scalar_kernel(const uint16_t* __restrict__ gate_up,
+                                                             const float* __restrict__ scale_tensor,
+                                                             uint8_t* __restrict__ output, uint16_t* __restrict__ next_buffer,
+                                                             int rows, int cols, int buffer_cols) {
+    const long total = (long)rows * cols;
+    const float s = scale_tensor[0];
+    const float inv_scale = (s != 0.f) ? 1.f / s : 1.f;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long r = i / cols;
+        const int c = (int)(i - r * cols);
+        const float g = load16<DT>(gate_up[r * 2 * cols + c]);
+        const float u = load16<DT>(gate_up[r * 2 * cols + cols + c]);
+        output[i] = cvt_fp8(silu_mul(g, u, inv_scale));
+    }
+    zero_next_buffer(next_buffer, (long)rows * buffer_cols);
+}
+
+}  // namespace hfrk
+
+extern "C" int hfrk_swiglu(const void* gate_up, const float* scale_tensor, void* output, void* next_buffer, int rows,
+                           int cols, int buffer_cols, int io_dtype, int num_threads, int force_scalar, void* stream) {
+    using namespace hfrk;
+    if (rows < 0 || cols < 1 || buffer_cols < 0) return HFRK_BAD_SHAPE;
+    if (rows == 0) return HFRK_SUCCESS;
+    if (!gate_up || !scale_tensor || !output) return HFRK_BAD_SHAPE;
+    if (buffer_cols > 0 && !next_buffer) return HFRK_BAD_SHAPE;
+    if (io_dtype != HFRK_F16 && io_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
+    if (num_threads < 0 || num_threads > 1024) return HFRK_INVALID_CONFIG;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint16_t* in = static_cast<const uint16_t*>(gate_up);
+    uint8_t* out = static_cast<uint8_t*>(output);
+    uint16_t* nb = static_cast<uint16_t*>(next_buffer);
+    const bool vec = !force_scalar && (cols % 8 == 0) && (reinterpret_cast<uintptr_t>(gate_up) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(output) & 7) == 0;
+    int threads = num_threads > 0 ? num_threads : 256;
+    const long work = vec ? (long)rows * (cols / 8) : (long)rows * cols;
+    long blocks = (work + threads - 1) / threads;
+    // enough workgroups to cover the chip a few times over; the loop in the kernel strides over the rest
+    const long cap = (long)kNumCU * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    if (io_dtype == HFRK_F16) {
+        if (vec) hipLaunchKernelGGL((swiglu_vec_kernel<HFRK_F16>), dim3((unsigned)blocks), dim3(threads), 0, s, in, scale_tensor, out, nb, rows, cols, buffer_cols);
+        else hipLaunchKernelGGL((swiglu_scalar_kernel<HFRK_F16>), dim3((unsigned)blocks), dim3(threads), 0, s, in, scale_tensor, out, nb, rows, cols, buffer_cols);
+    } else {
+        if (vec) hipLaunchKernelGGL((swiglu_vec_kernel<HFRK_BF16>), dim3((unsigned)blocks), dim3(threads), 0, s, in, scale_tensor, out, nb, rows, cols, buffer_cols);
+        else hipLaunchKernelGGL((swiglu_scalar_kernel<HFRK_BF16>), dim3((unsigned)blocks), dim3(threads), 0, s, in, scale_tensor, out, nb, rows, cols, buffer_cols);
+    }
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}

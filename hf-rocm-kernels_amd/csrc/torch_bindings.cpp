@@ -1,0 +1,203 @@
+// torch.ops._HFRK_C.* -- the operator surface of the reference (csrc/torch_bindings.cpp:20-44, csrc/ops.h:8-19),
+// same schemas, implemented by forwarding plain pointers to the C ABI of libhfrk_gfx950.so.
+// No kernel lives here: this file only unpacks tensors, checks them, selects device and stream.
+#include <Python.h>
+
+#include <ATen/ATen.h>
+#include <c10/hip/HIPFunctions.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include "hfrk_gfx950.h"
+
+namespace {
+
+// Make the tensor's device current for the duration of a call (the launchers use the current device).
+struct DeviceScope {
+    c10::DeviceIndex prev;
+    bool changed;
+    explicit DeviceScope(const at::Tensor& t) : prev(c10::hip::current_device()), changed(false) {
+        const c10::DeviceIndex want = t.device().index();
+        if (want >= 0 && want != prev) {
+            c10::hip::set_device(want);
+            changed = true;
+        }
+    }
+    ~DeviceScope() {
+        if (changed) c10::hip::set_device(prev);
+    }
+};
+
+void* current_stream(const at::Tensor& t) {
+    return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+int dtype16(const at::Tensor& t, const char* name) {
+    if (t.scalar_type() == at::kBFloat16) return HFRK_BF16;
+    if (t.scalar_type() == at::kHalf) return HFRK_F16;
+    TORCH_CHECK(false, name, " must be float16 or bfloat16, got ", t.scalar_type());
+}
+
+void check_fp8(const at::Tensor& t, const char* name) {
+    TORCH_CHECK(t.scalar_type() != at::kFloat8_e4m3fnuz, name,
+                " is float8_e4m3fnuz: gfx950 computes in OCP float8_e4m3fn (same bits read as twice the fnuz value); "
+                "re-encode the tensor or pass a float8_e4m3fn view and double its scale");
+    TORCH_CHECK(t.scalar_type() == at::kFloat8_e4m3fn, name, " must be float8_e4m3fn, got ", t.scalar_type());
+}
+
+void check_same_device(const at::Tensor& ref, const at::Tensor& t, const char* name) {
+    TORCH_CHECK(t.device() == ref.device(), name, " is on ", t.device(), " but expected ", ref.device());
+}
+
+void raise_on(int status, const char* op) {
+    TORCH_CHECK(status == HFRK_SUCCESS, op, " failed: ", hfrk_status_string(status), " (status ", status,
+                ", hip error ", hfrk_last_hip_error(), ")");
+}
+
+// reference: csrc/op_src/increment/increment_op.cu:3
+void increment(at::Tensor& x) { x += 1; }
+
+// reference: csrc/op_src/residual_rms/residual_rms_dispatch.cu:8-63
+void residual_rms(at::Tensor& input, at::Tensor& residual, at::Tensor& weight, at::Tensor& scale_tensor, double epsilon,
+                  at::Tensor& output, at::Tensor& next_buffer, int64_t num_threads, bool force_scalar) {
+    TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous [rows, cols] tensor");
+    TORCH_CHECK(residual.sizes() == input.sizes() && residual.is_contiguous(), "residual must match input and be contiguous");
+    TORCH_CHECK(weight.dim() == 1 && weight.size(0) == input.size(1) && weight.is_contiguous(), "weight must be [cols]");
+    TORCH_CHECK(output.sizes() == input.sizes() && output.is_contiguous(), "output must match input and be contiguous");
+    const int io = dtype16(input, "input");
+    TORCH_CHECK(residual.scalar_type() == input.scalar_type() && weight.scalar_type() == input.scalar_type(),
+                "input, residual and weight must share one 16-bit dtype");
+    int out = io;
+    if (output.scalar_type() != input.scalar_type()) {
+        check_fp8(output, "output");
+        out = HFRK_FP8_E4M3FN;
+        TORCH_CHECK(scale_tensor.numel() == 1 && scale_tensor.scalar_type() == at::kFloat, "fp8 output needs a one-element float32 scale_tensor");
+        check_same_device(input, scale_tensor, "scale_tensor");
+    }
+    check_same_device(input, residual, "residual");
+    check_same_device(input, weight, "weight");
+    check_same_device(input, output, "output");
+    int64_t buffer_cols = 0;
+    void* nb = nullptr;
+    if (next_buffer.numel() > 0) {
+        TORCH_CHECK(next_buffer.dim() == 2 && next_buffer.size(0) == input.size(0) && next_buffer.is_contiguous(),
+                    "next_buffer must be a contiguous [rows, buffer_cols] tensor");
+        TORCH_CHECK(next_buffer.element_size() == 2, "next_buffer must hold 16-bit elements");
+        check_same_device(input, next_buffer, "next_buffer");
+        buffer_cols = next_buffer.size(1);
+        nb = next_buffer.data_ptr();
+    }
+    DeviceScope scope(input);
+    raise_on(hfrk_residual_rms(input.data_ptr(), residual.data_ptr(), weight.data_ptr(),
+                               out == HFRK_FP8_E4M3FN ? scale_tensor.data_ptr<float>() : nullptr, (float)epsilon,
+                               output.data_ptr(), nb, (int)input.size(0), (int)input.size(1), (int)buffer_cols, io, out,
+                               (int)num_threads, force_scalar ? 1 : 0, current_stream(input)),
+             "residual_rms");
+}
+
+// reference: csrc/op_src/swiglu/swiglu_dispatch.cu:8-42
+void swiglu(at::Tensor& gate_up, at::Tensor& scale_tensor, at::Tensor& output, at::Tensor& next_buffer, int64_t num_threads,
+            bool force_scalar) {
+    TORCH_CHECK(gate_up.dim() == 2 && gate_up.is_contiguous() && gate_up.size(1) % 2 == 0,
+                "gate_up must be a contiguous [rows, 2*cols] tensor");
+    const int io = dtype16(gate_up, "gate_up");
+    const int64_t rows = gate_up.size(0), cols = gate_up.size(1) / 2;
+    check_fp8(output, "output");
+    TORCH_CHECK(output.dim() == 2 && output.size(0) == rows && output.size(1) == cols && output.is_contiguous(),
+                "output must be a contiguous [rows, cols] tensor");
+    TORCH_CHECK(scale_tensor.numel() == 1 && scale_tensor.scalar_type() == at::kFloat, "scale_tensor must be one float32");
+    check_same_device(gate_up, scale_tensor, "scale_tensor");
+    check_same_device(gate_up, output, "output");
+    int64_t buffer_cols = 0;
+    void* nb = nullptr;
+    if (next_buffer.numel() > 0) {
+        TORCH_CHECK(next_buffer.dim() == 2 && next_buffer.size(0) == rows && next_buffer.is_contiguous(),
+                    "next_buffer must be a contiguous [rows, buffer_cols] tensor");
+        TORCH_CHECK(next_buffer.element_size() == 2, "next_buffer must hold 16-bit elements");
+        check_same_device(gate_up, next_buffer, "next_buffer");
+        buffer_cols = next_buffer.size(1);
+        nb = next_buffer.data_ptr();
+    }
+    DeviceScope scope(gate_up);
+    raise_on(hfrk_swiglu(gate_up.data_ptr(), scale_tensor.data_ptr<float>(), output.data_ptr(), nb, (int)rows, (int)cols,
+                         (int)buffer_cols, io, (int)(num_threads < 0 ? 0 : num_threads), force_scalar ? 1 : 0,
+                         current_stream(gate_up)),
+             "swiglu");
+}
+
+void check_gemm_operands(const at::Tensor& A, const at::Tensor& B, const at::Tensor& D) {
+    TORCH_CHECK(A.dim() == 2 && A.is_contiguous(), "A must be a contiguous [m, k] tensor");
+    TORCH_CHECK(B.dim() == 2 && B.size(0) == A.size(1) && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
+    TORCH_CHECK(D.dim() == 2 && D.size(0) == A.size(0) && D.size(1) == B.size(1) && D.is_contiguous(),
+                "D must be a contiguous [m, n] tensor");
+    check_fp8(A, "A");
+    check_fp8(B, "B");
+    check_same_device(A, B, "B");
+    check_same_device(A, D, "D");
+}
+
+// reference: csrc/op_src/skinny_gemm/skinny_gemm_binding.cu:16-42.  Returns the status code like the reference;
+// misuse of dtypes/devices raises instead of reading garbage.
+int64_t skinny_gemm_tb(at::Tensor& A, at::Tensor& B, at::Tensor& D, at::Tensor& scale_tensor, int64_t split_k,
+                       int64_t A_producers, int64_t B_producers, int64_t consumers, int64_t a_lanes, int64_t b_lanes,
+                       int64_t qsize, int64_t op_m, int64_t ops) {
+    check_gemm_operands(A, B, D);
+    TORCH_CHECK(scale_tensor.numel() == 1 && scale_tensor.scalar_type() == at::kFloat, "scale_tensor must be one float32");
+    check_same_device(A, scale_tensor, "scale_tensor");
+    const int d_dtype = dtype16(D, "D");
+    DeviceScope scope(A);  // before the stream is looked up
+    return hfrk_skinny_gemm(A.data_ptr(), B.data_ptr(), D.data_ptr(), scale_tensor.data_ptr<float>(), (int)A.size(0),
+                            (int)B.size(1), (int)A.size(1), (int)B.stride(1), (int)split_k, (int)A_producers,
+                            (int)B_producers, (int)consumers, (int)a_lanes, (int)b_lanes, (int)qsize, (int)op_m, (int)ops,
+                            d_dtype, current_stream(A));
+}
+
+// Per-token (scale_a: 1 or m values) x per-output-channel (scale_b: 1 or n values) scaling.  No reference counterpart.
+int64_t skinny_gemm_scaled(at::Tensor& A, at::Tensor& B, at::Tensor& D, at::Tensor& scale_a, at::Tensor& scale_b,
+                           bool accumulate) {
+    check_gemm_operands(A, B, D);
+    const int64_t m = A.size(0), n = B.size(1);
+    TORCH_CHECK(scale_a.scalar_type() == at::kFloat && scale_a.is_contiguous() && (scale_a.numel() == 1 || scale_a.numel() == m),
+                "scale_a must be float32 with 1 or m elements");
+    TORCH_CHECK(scale_b.scalar_type() == at::kFloat && scale_b.is_contiguous() && (scale_b.numel() == 1 || scale_b.numel() == n),
+                "scale_b must be float32 with 1 or n elements");
+    check_same_device(A, scale_a, "scale_a");
+    check_same_device(A, scale_b, "scale_b");
+    const int d_dtype = dtype16(D, "D");
+    DeviceScope scope(A);
+    return hfrk_skinny_gemm_ex(A.data_ptr(), B.data_ptr(), D.data_ptr(), scale_a.data_ptr<float>(),
+                               scale_a.numel() == 1 ? 0 : 1, scale_b.data_ptr<float>(), scale_b.numel() == 1 ? 0 : 1, (int)m,
+                               (int)n, (int)A.size(1), (int)B.stride(1), d_dtype, accumulate ? 1 : 0, nullptr,
+                               current_stream(A));
+}
+
+}  // namespace
+
+TORCH_LIBRARY(_HFRK_C, ops) {
+    ops.def("increment(Tensor! x) -> ()");
+    ops.impl("increment", c10::kCUDA, &increment);
+
+    ops.def(
+        "residual_rms(Tensor input, Tensor! residual, Tensor weight, Tensor scale_tensor, float epsilon, Tensor! "
+        "output, Tensor! next_buffer, int num_threads, bool force_scalar) -> ()");
+    ops.impl("residual_rms", c10::kCUDA, &residual_rms);
+
+    ops.def(
+        "swiglu(Tensor gate_up, Tensor scale_tensor, Tensor! output, Tensor! next_buffer, int num_threads, "
+        "bool force_scalar) -> ()");
+    ops.impl("swiglu", c10::kCUDA, &swiglu);
+
+    ops.def(
+        "skinny_gemm_tb(Tensor A, Tensor B, Tensor! D, Tensor scale_tensor, int split_k, int A_producers, "
+        "int B_producers, int consumers, int a_lanes, int b_lanes, int qsize, int op_m, int ops) -> int");
+    ops.impl("skinny_gemm_tb", c10::kCUDA, &skinny_gemm_tb);
+
+    ops.def("skinny_gemm_scaled(Tensor A, Tensor B, Tensor! D, Tensor scale_a, Tensor scale_b, bool accumulate) -> int");
+    ops.impl("skinny_gemm_scaled", c10::kCUDA, &skinny_gemm_scaled);
+}
+
+// `import hf_rocm_kernels._HFRK_C` loads this library and thereby runs the registration above.
+PyMODINIT_FUNC PyInit__HFRK_C(void) {
+    static struct PyModuleDef module = {PyModuleDef_HEAD_INIT, "_HFRK_C", nullptr, 0, nullptr};
+    return PyModule_Create(&module);
+}

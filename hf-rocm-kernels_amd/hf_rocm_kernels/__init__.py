@@ -1,0 +1,12 @@
+"""MI355X (gfx950) implementation of the `hf_rocm_kernels` operator surface.
+
+Same names as the reference package (hf_rocm_kernels/__init__.py:1-6): four operators backed by
+`torch.ops._HFRK_C`, which forwards to the C ABI of `libhfrk_gfx950.so` (include/hfrk_gfx950.h).
+Importing this package loads both shared objects and fails if either is missing: there is no fallback path.
+"""
+from .operators.increment import increment
+from .operators.residual_rms import residual_rms
+from .operators.swiglu import swiglu
+from .operators.skinny_gemm import skinny_gemm, skinny_gemm_scaled
+
+__all__ = ["increment", "residual_rms", "swiglu", "skinny_gemm", "skinny_gemm_scaled"]

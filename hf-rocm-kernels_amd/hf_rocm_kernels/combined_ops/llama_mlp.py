@@ -1,0 +1,65 @@
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from hf_rocm_kernels import residual_rms, skinny_gemm, swiglu
+
+
+def llama_mlp_combined_ops(
+    attn_output: Tensor,
+    residual: Tensor,
+    rms_weight: Tensor,
+    rms_epsilon: float,
+    gate_up_weight: Tensor,
+    gate_up_input_scale: Tensor,
+    gate_up_output_scale: Tensor,
+    down_weight: Tensor,
+    down_input_scale: Tensor,
+    down_output_scale: Tensor,
+    gate_up_gemm_hp: Tuple[Optional[int], Optional[int]] = (None, None),
+    down_gemm_hp: Tuple[Optional[int], Optional[int]] = (None, None),
+    add_residual: bool = False,
+) -> Tuple[Tensor, Tensor]:
+    """Decoder MLP sub-block as four launches on one stream (reference: combined_ops/llama_mlp.py:7-60):
+    residual RMSNorm -> fp8, gate_up GEMM, SwiGLU -> fp8, down GEMM.
+
+    - attn_output, residual: (m, hidden) 16-bit; residual <- attn_output + residual in place
+    - gate_up_weight: (hidden, 2*inter) fp8, col-major; down_weight: (inter, hidden) fp8, col-major
+    - *_input_scale: the activation quantisation scale of each GEMM; *_output_scale: activation scale x weight scale
+    - gate_up_gemm_hp / down_gemm_hp: accepted for signature compatibility; the library plans each GEMM itself
+      (the reference forwards them as split_k / b_lanes keywords its skinny_gemm does not take)
+    - add_residual: the down projection accumulates onto a copy of the updated residual instead of zeros, so
+      the first output is the block's output hidden state (residual + mlp) rounded once
+
+    RMSNorm and SwiGLU zero the buffer the following GEMM accumulates into, as in the reference.
+    Returns (mlp_output, residual)."""
+    del gate_up_gemm_hp, down_gemm_hp
+    m = attn_output.size(0)
+    dtype = attn_output.dtype
+
+    # RMS norm (zeroes the gate_up GEMM's accumulator)
+    gate_up_proj = torch.empty(size=(m, gate_up_weight.size(1)), dtype=dtype, device=attn_output.device)
+    normalized, residual = residual_rms(
+        input=attn_output,
+        residual=residual,
+        weight=rms_weight,
+        epsilon=rms_epsilon,
+        scale_tensor=gate_up_input_scale,
+        next_buffer=gate_up_proj,
+    )
+
+    # Gate + up projection
+    skinny_gemm(skinny_a=normalized, b=gate_up_weight, scale_tensor=gate_up_output_scale, output=gate_up_proj)
+
+    # Swiglu (zeroes the down GEMM's accumulator unless it starts from the residual)
+    if add_residual:
+        mlp_output = residual.clone()
+        swiglu_out = swiglu(gate_up_proj=gate_up_proj, scale_tensor=down_input_scale)
+    else:
+        mlp_output = torch.empty(size=(m, down_weight.size(1)), dtype=dtype, device=attn_output.device)
+        swiglu_out = swiglu(gate_up_proj=gate_up_proj, scale_tensor=down_input_scale, next_buffer=mlp_output)
+
+    # Down projection
+    skinny_gemm(skinny_a=swiglu_out, b=down_weight, scale_tensor=down_output_scale, output=mlp_output)
+    return mlp_output, residual

@@ -1,0 +1,4 @@
+from .wrapped import skinny_gemm, skinny_gemm_scaled
+from .data import generate_skinny_gemm_data, generate_llama_gemm_data
+
+__all__ = ["skinny_gemm", "skinny_gemm_scaled", "generate_skinny_gemm_data", "generate_llama_gemm_data"]

@@ -1,0 +1,120 @@
+from typing import Dict, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from ... import _capi
+from .binding import _skinny_gemm, _skinny_gemm_scaled
+
+_OUT_DTYPES = (torch.bfloat16, torch.float16)
+
+
+def skinny_gemm_checks(
+    skinny_a: Tensor,
+    b: Tensor,
+    scale_tensor: Tensor,
+    output: Tensor,
+) -> None:
+    """Same assertions as the reference (operators/skinny_gemm/wrapped.py:9-35), with the dtypes of this build:
+    float8_e4m3fn operands (gfx950 is OCP fp8, not fnuz) and a bfloat16 or float16 output."""
+    # Check shapes
+    assert skinny_a.dim() == 2, f"Expected skinny_a to have 2 dimensions but got {skinny_a.dim() = } instead."
+    assert skinny_a.size(1) == b.size(0), f"Expected {skinny_a.size(1) = } and {b.size(0) = } to be the same."
+    assert scale_tensor.numel() == 1, f"Expected {scale_tensor.numel() = } to be 1."
+    assert output.shape == (skinny_a.size(0), b.size(1)), (
+        f"{output.shape} does not match with {skinny_a.shape = } and {b.shape =}")
+    # Check layouts
+    assert skinny_a.is_contiguous(), f"Expected skinny_a to be contiguous but got {skinny_a.stride() = }"
+    assert b.stride(0) == 1, f"Expected b to be column-major but got {b.stride() = }"
+    assert output.is_contiguous(), f"Expected output to be contiguous but got {output.stride() = }"
+    # Check dtypes
+    assert skinny_a.dtype == torch.float8_e4m3fn, f"Expected {skinny_a.dtype = } to be torch.float8_e4m3fn"
+    assert b.dtype == torch.float8_e4m3fn, f"Expected {b.dtype = } to be torch.float8_e4m3fn"
+    assert scale_tensor.dtype == torch.float32, f"Expected {scale_tensor.dtype = } to be torch.float32"
+    assert output.dtype in _OUT_DTYPES, f"Expected {output.dtype = } to be torch.bfloat16 or torch.float16"
+    # Check devices
+    device = skinny_a.device
+    assert device.type == "cuda", f"Expected input.device to be of type cuda, but got {device.type = } instead."
+    assert b.device == device, f"Expected {b.device = } to be the same as {device = }"
+    assert scale_tensor.device == device, f"Expected {scale_tensor.device = } to be the same as {device = }"
+    assert output.device == device, f"Expected {output.device = } to be the same as {device = }"
+
+
+def infer_skinny_gemm_m_params(m: int) -> Tuple[int, int]:
+    """(a_lanes, op_m) exactly as the reference derives them from m (wrapped.py:37-40)."""
+    a_lanes = 2 if m > 16 else 1
+    op_m = 16 if m > 8 else 8
+    return a_lanes, op_m
+
+
+def infer_skinny_gemm_params(skinny_a: Tensor, b: Tensor) -> Dict[str, int]:
+    """The nine integers of the op schema.
+
+    The reference looks them up in a table tuned for four shapes on 304 CUs (wrapped.py:42-102).  Here the
+    decomposition is chosen by the library's planner (`hfrk_skinny_gemm_plan`, one persistent workgroup per CU
+    of 256, stream-K over (row panel, K slab) units); the integers only have to pass the launcher's validation,
+    so they are the reference's defaults, with `split_k` reporting the planner's K slabs per panel."""
+    m, k = skinny_a.shape
+    n = b.shape[1]
+    a_lanes, op_m = infer_skinny_gemm_m_params(m)
+    ops = 4 if op_m == 8 else 8
+    b_lanes = min(4, max(1, n // (256 * 16)))
+    qsize = 3
+    plan = _capi.plan(m, n, k)
+    return {"A_producers": 3, "B_producers": min(6, qsize * b_lanes), "consumers": 3,
+            "a_lanes": a_lanes, "b_lanes": b_lanes,
+            "qsize": qsize, "op_m": op_m, "ops": ops, "split_k": plan.slabs}
+
+
+def _raise_on_status(status: int, what: str) -> None:
+    if status != _capi.SUCCESS:
+        raise RuntimeError(f"{what} rejected the call with status {status}: {_capi.status_string(status)}")
+
+
+def skinny_gemm(
+    skinny_a: Tensor,
+    b: Tensor,
+    scale_tensor: Tensor,
+    output: Optional[Tensor] = None,
+) -> Tensor:
+    """FP8 skinny GEMM: output += scale * skinny_a @ b, fp32 accumulation, one rounding.
+    Args (reference: operators/skinny_gemm/wrapped.py:104-128):
+        - skinny_a: a float8_e4m3fn tensor of shape (m, k) in row-major format, m <= 64
+        - b: a float8_e4m3fn tensor of shape (k, n) in col-major format (an nn.Linear weight [n, k], transposed)
+        - scale_tensor: a fp32 one-item tensor, the product of the two quantisation scales
+        - output: an optional (m, n) bfloat16/float16 tensor that is accumulated into: zero-initialised, or
+          holding a bias or residual.  Allocated as bfloat16 zeros when omitted.
+    Outputs:
+        the (m, n) output tensor.
+    Unlike the reference, a launcher status other than 0 raises instead of leaving the output untouched.
+    """
+    if output is None:
+        output = torch.zeros(size=(skinny_a.size(0), b.size(1)), dtype=torch.bfloat16, device=skinny_a.device)
+    skinny_gemm_checks(skinny_a, b, scale_tensor, output)
+    kwargs = infer_skinny_gemm_params(skinny_a, b)
+    status = _skinny_gemm(A=skinny_a, B=b, scale_tensor=scale_tensor, D=output, **kwargs)
+    _raise_on_status(status, "skinny_gemm_tb")
+    return output
+
+
+def skinny_gemm_scaled(
+    skinny_a: Tensor,
+    b: Tensor,
+    scale_a: Tensor,
+    scale_b: Tensor,
+    output: Optional[Tensor] = None,
+    accumulate: bool = False,
+) -> Tensor:
+    """Per-token x per-output-channel variant: output[i, j] (+)= scale_a[i] * scale_b[j] * (skinny_a @ b)[i, j].
+    `scale_a` has 1 or m float32 elements, `scale_b` 1 or n.  With accumulate=False the output is overwritten."""
+    m, n = skinny_a.size(0), b.size(1)
+    if output is None:
+        output = torch.empty(size=(m, n), dtype=torch.bfloat16, device=skinny_a.device)
+        accumulate = False
+    skinny_gemm_checks(skinny_a, b, scale_a.reshape(-1)[:1], output)
+    assert scale_a.numel() in (1, m) and scale_a.dtype == torch.float32, f"Expected 1 or {m} float32 in scale_a"
+    assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
+    status = _skinny_gemm_scaled(skinny_a, b, output, scale_a.contiguous().view(-1), scale_b.contiguous().view(-1),
+                                 accumulate)
+    _raise_on_status(status, "skinny_gemm_scaled")
+    return output

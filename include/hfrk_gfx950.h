@@ -1,0 +1,126 @@
+/*
+ * hfrk_gfx950.h -- C ABI of libhfrk_gfx950.so: FP8 skinny GEMM, residual RMSNorm and SwiGLU for MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; every pointer is a DEVICE pointer unless stated otherwise, every call is
+ * asynchronous on `stream` (a hipStream_t passed as void*; NULL = the default stream) and launches on the
+ * device that is current on the calling thread.  No call synchronises, reads back, or (after hfrk_init for
+ * that device) allocates, so all of them can be recorded into a HIP graph.
+ *
+ * FP8 is OCP e4m3fn (bias 7, max 448, no infinities) -- the format gfx950's matrix cores implement.  The
+ * reference was written for gfx942's e4m3fnuz; on the same bits an fnuz value is half the fn value.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the reference tree).
+ */
+#ifndef HFRK_GFX950_H
+#define HFRK_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  0..6 are the reference's SkinnyGemmReturnCode (csrc/op_src/skinny_gemm/skinny_gemm_caller.cu:9-17),
+ * same numbers, same conditions; the rest are additions of this library. */
+enum hfrk_status {
+    HFRK_SUCCESS = 0,
+    HFRK_M_ABOVE_WARPTILE_M = 1,            /* never returned (the reference has the check commented out) */
+    HFRK_N_NOT_EVEN = 2,
+    HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K = 3, /* k % ((512/op_m)*ops) != 0, or k % 256 != 0 */
+    HFRK_TOO_MANY_WARPS = 4,                /* A_producers + B_producers + consumers > 16 */
+    HFRK_QSIZE_TOO_SMALL = 5,
+    HFRK_INVALID_CONFIG = 6,                /* knob tuple outside the accepted domain */
+    HFRK_BAD_SHAPE = 7,                     /* m < 1, m > 64, n < 1, k < 1, extent over 2 GiB ... */
+    HFRK_BAD_ALIGNMENT = 8,                 /* a pointer or stride that must be 16-byte aligned is not */
+    HFRK_BAD_DTYPE = 9,
+    HFRK_HIP_ERROR = 10,                    /* a HIP runtime call failed; hfrk_last_hip_error() has the code */
+    HFRK_NOT_INITIALISED = 11               /* workspace missing and the stream is capturing (call hfrk_init first) */
+};
+
+/* Element types of 16-bit tensors. */
+enum hfrk_dtype { HFRK_F16 = 0, HFRK_BF16 = 1, HFRK_FP8_E4M3FN = 2 };
+
+/* Largest m the skinny GEMM accepts. */
+#define HFRK_GEMM_MAX_M 64
+
+/* How one GEMM call is decomposed.  Filled by hfrk_skinny_gemm_plan(); may be edited and passed back to
+ * hfrk_skinny_gemm_ex() by an autotuner (counterpart of the knob table in
+ * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102 and benchmarks/skinny_gemm/grid_search.py). */
+typedef struct hfrk_gemm_plan {
+    int m_tiles;   /* ceil(m/16): 16-row activation tiles kept in registers (1..4) */
+    int wn;        /* waves of a workgroup spread over output rows (16 weight rows each) */
+    int wk;        /* waves of a workgroup spread over K; wn*wk = 8 waves */
+    int ch;        /* 256-byte K chunks each wave streams per slab (1 or 2) */
+    int grid;      /* persistent workgroups launched (<= 256, one per CU) */
+    int panels;    /* ceil(n / (16*wn)) */
+    int slabs;     /* k / (256*wk*ch): K slabs per panel */
+    int lds_bytes; /* dynamic LDS per workgroup */
+} hfrk_gemm_plan;
+
+/* Library version, for the binding to check. */
+int hfrk_version(void);
+
+/* Allocate (once per device) the split-K workspace of the current device.  Idempotent, thread-safe.
+ * Must have run on a device before a GEMM on that device is captured into a graph.  No reference counterpart
+ * (the reference accumulates with fp16 atomics into a caller-zeroed output instead of using a workspace). */
+int hfrk_init(void);
+
+/* hipError_t of the last failed HIP call on this thread (0 if none). */
+int hfrk_last_hip_error(void);
+
+/* Human-readable text for a status code (static storage). */
+const char* hfrk_status_string(int status);
+
+/* Pure host function: the reference launcher's argument checks, same order, same codes
+ * (csrc/op_src/skinny_gemm/skinny_gemm_caller.cu:33-72,455-457), plus this library's own shape limits.
+ * Touches no device. */
+int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, int A_producers, int B_producers,
+                              int consumers, int a_lanes, int b_lanes, int qsize, int op_m, int ops);
+
+/* Pure host function: choose the decomposition for a shape (counterpart of infer_skinny_gemm_params,
+ * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102).  Returns HFRK_SUCCESS or a shape error. */
+int hfrk_skinny_gemm_plan(int m, int n, int k, hfrk_gemm_plan* plan);
+
+/* D[m,n] += scale_tensor[0] * A[m,k] . B[k,n]
+ * Replaces `int skinny_gemm(...)` at csrc/op_src/skinny_gemm/skinny_gemm_caller.cu:21-32, the function behind
+ * torch.ops._HFRK_C.skinny_gemm_tb (csrc/op_src/skinny_gemm/skinny_gemm_binding.cu:16-42), same argument order.
+ *   A   fp8 e4m3fn [m,k] row-major            B   fp8 e4m3fn [k,n] with unit stride along k: row n of the
+ *   D   16-bit [m,n] row-major, d_dtype           weight starts at B + n*b_stride (b_stride in elements)
+ *   scale_tensor  one fp32 (the product of the activation and weight scales)
+ * D is accumulated into, once, in fp32 (D = round(float(D) + scale*acc)): callers pre-zero it or preload a
+ * bias, as with the reference, but the result is deterministic and rounded a single time.
+ * split_k and the eight knob integers are validated exactly like the reference's and are otherwise advisory:
+ * the decomposition comes from hfrk_skinny_gemm_plan(). */
+int hfrk_skinny_gemm(const void* A, const void* B, void* D, const float* scale_tensor, int m, int n, int k,
+                     int b_stride, int split_k, int A_producers, int B_producers, int consumers, int a_lanes,
+                     int b_lanes, int qsize, int op_m, int ops, int d_dtype, void* stream);
+
+/* General form: D[i,j] = (accumulate ? D[i,j] : 0) + scale_a[i*sa_stride] * scale_b[j*sb_stride] * sum_k A[i,k] B[k,j]
+ * sa_stride / sb_stride are 0 (one scalar) or 1 (per token / per output channel).  scale_b may be NULL (= 1).
+ * plan may be NULL (the library plans).  No reference counterpart for the per-row/per-channel scales: the
+ * reference asserts scale_tensor.numel()==1 (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:18). */
+int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
+                        const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
+                        int accumulate, const hfrk_gemm_plan* plan, void* stream);
+
+/* residual <- input + residual (one 16-bit add); output <- rmsnorm(residual) * weight, optionally / scale -> fp8.
+ * Replaces `void residual_rms(...)` at csrc/op_src/residual_rms/residual_rms_dispatch.cu:8-63.
+ *   input, residual [rows,cols] io_dtype (f16/bf16) row-major; weight [cols] io_dtype
+ *   scale_tensor: one fp32, used (and required) only when out_dtype is fp8
+ *   output [rows,cols] out_dtype: HFRK_FP8_E4M3FN, or io_dtype
+ *   next_buffer: rows*buffer_cols 16-bit elements set to zero (may be NULL when buffer_cols==0)
+ *   num_threads: 0 = choose; else threads per row (multiple of 64, <= 1024).  force_scalar: use the
+ *   one-element-per-thread kernel even when the 16-byte path applies. */
+int hfrk_residual_rms(const void* input, void* residual, const void* weight, const float* scale_tensor,
+                      float epsilon, void* output, void* next_buffer, int rows, int cols, int buffer_cols,
+                      int io_dtype, int out_dtype, int num_threads, int force_scalar, void* stream);
+
+/* output[r,c] = fp8( silu(gate_up[r,c]) * gate_up[r,cols+c] / scale ), gate_up [rows, 2*cols] io_dtype.
+ * Replaces `void swiglu(...)` at csrc/op_src/swiglu/swiglu_dispatch.cu:8-42.  next_buffer as above. */
+int hfrk_swiglu(const void* gate_up, const float* scale_tensor, void* output, void* next_buffer, int rows,
+                int cols, int buffer_cols, int io_dtype, int num_threads, int force_scalar, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HFRK_GFX950_H */
