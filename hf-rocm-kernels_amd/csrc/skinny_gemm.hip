@@ -98,7 +98,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         saq[mt] = a.scale_a[(long)mrow * a.sa_stride];
     }
     const bool n_vec = (a.n & 3) == 0;
-    auto panel_fetch = [&](int panel, uint2 (&dd)[MT], float (&sb)[4]) {
+    auto panel_fetch = [&](int panel, uint2 (&dd)[MT], float (&sb)[4]) __attribute__((always_inline)) {
         const int n0 = panel * BN + wn * 16 + 4 * lg;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -129,11 +129,18 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
     v4i wq[2][CH][4];
     int ip = u0 / S, is = u0 % S;  // (panel, slab) of the next unit to issue
+    // Panel p walks its K slabs starting from slab p % S (sums do not care about the order): workgroups that move
+    // through their panels in step then read different activation slabs at any moment instead of all hitting
+    // the same few L2 lines.
+    auto phys_slab = [&](int panel, int slab) __attribute__((always_inline)) {
+        const int r = slab + panel % S;
+        return r >= S ? r - S : r;
+    };
     bool issue_first = true;       // next unit to issue opens a panel for this workgroup
     // Every step issues the same number of loads, in range or not: a unit past the end of this workgroup's range
     // is requested at an offset beyond the buffer, which returns zeros without touching memory.  That keeps the
     // count of loads in flight a compile-time constant, so each wait leaves exactly the prefetched unit pending.
-    auto issue_unit = [&](auto sel, bool in_range) {
+    auto issue_unit = [&](auto sel, bool in_range) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
         if (in_range && issue_first) {
             if (wk == 0) {
@@ -144,7 +151,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         }
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)is * KS +
+            const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
                                                  (uint32_t)(c * WK + wk) * 256u
                                            : 0x80000000u;
 #pragma unroll
@@ -158,8 +165,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 
     // ---- activation slab staging ---------------------------------------------------------------------------
     v4i aq[APT];
-    auto act_load = [&](int slab, bool in_range) {
-        const uint32_t base = in_range ? (uint32_t)slab * KS : 0x80000000u;
+    // always called just before issue_unit for the same unit, so (ip, is) name that unit
+    auto act_load = [&](bool in_range) __attribute__((always_inline)) {
+        uint32_t base = in_range ? (uint32_t)phys_slab(ip, is) * KS : 0x80000000u;
+#ifdef HFRK_EXP_NOACT  // measurement only: request nothing, results are wrong
+        base = 0x80000000u;
+#endif
 #pragma unroll
         for (int q = 0; q < APT; ++q) {
             const int idx = tid + q * kGemmThreads;
@@ -170,7 +181,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             }
         }
     };
-    auto act_store = [&](int buf) {
+    auto act_store = [&](int buf) __attribute__((always_inline)) {
         uint8_t* const dst = act_all + buf * ACT_BYTES;
 #pragma unroll
         for (int q = 0; q < APT; ++q) {
@@ -198,7 +209,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 #pragma unroll
     for (int h = 0; h < 2; ++h) rd_off[h] = ((((8 * h + 2 * lg) ^ li) & 15) << 4);  // piece 8h+2g; its pair is ^16
 
-    auto consume_unit = [&](auto sel, int buf) {
+    auto consume_unit = [&](auto sel, int buf) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
         const uint8_t* const act = act_all + buf * ACT_BYTES;
 #pragma unroll
@@ -230,7 +241,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 
     // ---- epilogue ------------------------------------------------------------------------------------------
     // lane holds, per m-tile, D^T[n0 + v][mt*16 + li], v = 0..3: scale, add the fetched D, round once, store
-    auto store_panel = [&](int panel, int par) {
+    auto store_panel = [&](int panel, int par) __attribute__((always_inline)) {
         const int n0 = panel * BN + wn * 16 + 4 * lg;
         const bool vec_ok = n_vec && (n0 + 3 < a.n);
 #pragma unroll
@@ -243,8 +254,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const float r = acc[mt][v] * (saq[mt] * (par ? sbq[1][v] : sbq[0][v]));
-                if (a.d_dtype == HFRK_BF16) o[v] = store16<HFRK_BF16>(a.accumulate ? load16<HFRK_BF16>((uint16_t)oe[v]) + r : r);
-                else o[v] = store16<HFRK_F16>(a.accumulate ? load16<HFRK_F16>((uint16_t)oe[v]) + r : r);
+                const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)oe[v]) : load16<HFRK_F16>((uint16_t)oe[v]);
+                const float sum = a.accumulate ? base + r : r;
+                o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
             }
             uint16_t* const drow = D + (long)mrow * a.n;
             if (vec_ok) {
@@ -257,14 +269,18 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         }
     };
 
-    // fp32 partial of (workgroup gg, slot): [wn][mt][lane] float4
-    auto ws_ptr = [&](int gg, int slot) -> v4f* {
-        return reinterpret_cast<v4f*>(a.ws) + ((size_t)(gg * 2 + slot) * (WN * MT)) * 64;
+    // fp32 partial of (workgroup gg, slot): [wn][mt][lane] float4.  Partials cross XCDs, whose L2s are not coherent
+    // with each other: they are written through to memory and read past the caches (sc0 sc1 on both sides), which
+    // keeps them coherent per location without the L2 write-back / invalidate a device-scope fence would cost.
+    const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
+    auto ws_off = [&](int gg, int slot, int mt) __attribute__((always_inline)) -> int {
+        return (((gg * 2 + slot) * (WN * MT) + wn * MT + mt) * 64 + lane) * 16;
     };
+    constexpr int kCoherent = 17;  // sc0 | sc1
 
     int flush_par = 0;  // context of the panel that closes next
     // close panel `panel`, of which this workgroup covered slabs [s_first, s_end)
-    auto flush_panel = [&](int panel, int s_first, int s_end) {
+    auto flush_panel = [&](int panel, int s_first, int s_end) __attribute__((always_inline)) {
         if constexpr (WK > 1) {
             // sum the WK waves that share rows; their transposition tiles are idle here and serve as scratch
             v4f* const mine = reinterpret_cast<v4f*>(tb);
@@ -289,10 +305,10 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         } else {
             const int slot = (panel == u0 / S) ? 0 : 1;
             if (wk == 0) {
-                v4f* const dst = ws_ptr(g, slot) + (wn * MT) * 64;
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) dst[mt * 64 + lane] = acc[mt];
-                __threadfence();
+                for (int mt = 0; mt < MT; ++mt)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, acc[mt]), ws_rsrc, ws_off(g, slot, mt), 0, kCoherent);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stores acknowledged before the arrival is counted
             }
             __syncthreads();
             if (tid == 0) {
@@ -305,7 +321,6 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             __syncthreads();
             const int last = *flag;
             if (last && wk == 0) {
-                __threadfence();
                 // contributors are the workgroups whose unit range meets [panel*S, (panel+1)*S), in id order
                 const long lo = (long)panel * S, hi = lo + S;
                 const int g_first = (int)(((lo + 1) * G + U - 1) / U) - 1;
@@ -314,9 +329,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                 for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
                 for (int gg = g_first; gg <= g_last; ++gg) {
                     const int sl = (unit_begin(gg, U, G) / S == panel) ? 0 : 1;
-                    const v4f* const src = ws_ptr(gg, sl) + (wn * MT) * 64;
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) acc[mt] += __builtin_nontemporal_load(src + mt * 64 + lane);
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt] += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_off(gg, sl, mt), 0, kCoherent));
                 }
                 store_panel(panel, flush_par);
             }
@@ -334,17 +349,17 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     using Sel1 = std::integral_constant<int, 1>;
     int cp = u0 / S, cs = u0 % S;  // (panel, slab) of the unit being consumed
     int s_first = cs;              // first slab this workgroup covers of the current panel
-    auto next_slab = [&](int s) { return (s + 1 == S) ? 0 : s + 1; };
+    auto next_slab = [&](int s) __attribute__((always_inline)) { return (s + 1 == S) ? 0 : s + 1; };
 
-    act_load(cs, true);
+    act_load(true);
     issue_unit(Sel0{}, true);
     act_store(0);
-    act_load(next_slab(cs), u0 + 1 < u1);
+    act_load(u0 + 1 < u1);
     issue_unit(Sel1{}, u0 + 1 < u1);
     __syncthreads();
 
     // One step = one unit.  A step whose unit lies past u1 (odd range length) multiplies zeros and changes nothing.
-    auto step = [&](auto sel, int u) {
+    auto step = [&](auto sel, int u) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
         const int ns = next_slab(cs);
         if (u + 1 < u1) act_store(X ^ 1);  // slab of unit u+1, requested one step ago
@@ -353,7 +368,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             flush_panel(cp, s_first, cs + 1);
             s_first = 0;
         }
-        act_load(next_slab(ns), u + 2 < u1);
+        act_load(u + 2 < u1);
         issue_unit(sel, u + 2 < u1);
         if (u + 1 < u1) __syncthreads();
         cs = ns;
@@ -409,9 +424,8 @@ static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
     return HFRK_SUCCESS;
 }
 
-static int lds_bytes_for(int mt, int wk, int ch) {
-    const int ks = 256 * wk * ch;
-    return kGemmWaves * kTileBytes + 2 * 16 * mt * ks + 16;
+constexpr int lds_bytes_for(int mt, int wk, int ch) {
+    return kGemmWaves * kTileBytes + 2 * 16 * mt * (256 * wk * ch) + 16;
 }
 
 // Rough time model of one candidate decomposition, in nanoseconds; only its ordering matters.
@@ -498,8 +512,11 @@ static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
 
 template <int MT>
 static int launch_mt(const GemmArgs& args, const hfrk_gemm_plan& p, hipStream_t stream) {
-#define HFRK_CASE(WN_, WK_, CH_) \
-    if (p.wn == WN_ && p.ch == CH_) return launch_one<MT, WN_, WK_, CH_>(args, p.lds_bytes, stream);
+    // decompositions whose activation slabs cannot fit in LDS are never planned and are not compiled
+#define HFRK_CASE(WN_, WK_, CH_)                                                             \
+    if constexpr (lds_bytes_for(MT, WK_, CH_) <= kLdsLimit) {                                \
+        if (p.wn == WN_ && p.ch == CH_) return launch_one<MT, WN_, WK_, CH_>(args, p.lds_bytes, stream); \
+    }
     HFRK_CASE(1, 8, 1) HFRK_CASE(1, 8, 2) HFRK_CASE(2, 4, 1) HFRK_CASE(2, 4, 2)
     HFRK_CASE(4, 2, 1) HFRK_CASE(4, 2, 2) HFRK_CASE(8, 1, 1) HFRK_CASE(8, 1, 2)
 #undef HFRK_CASE
