@@ -35,7 +35,8 @@ constexpr int kGemmThreads = kGemmWaves * kWave;
 constexpr int kTileBytes = 4096;                 // 16 rows x 256 B, one chunk of one wave
 constexpr int kLdsLimit = 160 * 1024;            // LDS per CU on gfx950
 constexpr int kMaxPanels = 1 << 20;              // per-panel arrival counters
-constexpr size_t kWsFloats = (size_t)2 * kNumCU * kGemmWaves * 4 * 256;  // 2 slots x grid x WN*MT KB (worst case)
+constexpr int kMaxGrid = 4 * kNumCU;              // persistent workgroups: up to 4 per CU when LDS and registers allow
+constexpr size_t kWsFloats = (size_t)2 * kMaxGrid * kGemmWaves * 4 * 256;  // 2 slots x grid x WN*MT KB (worst case)
 
 struct GemmArgs {
     const uint8_t* A;
@@ -140,8 +141,19 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // Every step issues the same number of loads, in range or not: a unit past the end of this workgroup's range
     // is requested at an offset beyond the buffer, which returns zeros without touching memory.  That keeps the
     // count of loads in flight a compile-time constant, so each wait leaves exactly the prefetched unit pending.
-    auto issue_unit = [&](auto sel, bool in_range) __attribute__((always_inline)) {
+    // Weight chunk c of unit (ip, is) into register set X.
+    auto issue_chunk = [&](auto sel, int c, bool in_range) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
+        const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
+                                             (uint32_t)(c * WK + wk) * 256u
+                                       : 0x80000000u;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(
+                w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+    };
+    // Epilogue inputs of unit (ip, is) if it opens a panel, then move on to the next unit.
+    auto issue_done = [&](bool in_range) __attribute__((always_inline)) {
         if (in_range && issue_first) {
             if (wk == 0) {
                 if (fetch_par) panel_fetch(ip, dq[1], sbq[1]);
@@ -149,18 +161,13 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             }
             fetch_par ^= 1;
         }
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
-                                                 (uint32_t)(c * WK + wk) * 256u
-                                           : 0x80000000u;
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(
-                    w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
-        }
         issue_first = false;
         if (++is == S) { is = 0; ++ip; issue_first = true; }
+    };
+    auto issue_unit = [&](auto sel, bool in_range) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c) issue_chunk(sel, c, in_range);
+        issue_done(in_range);
     };
 
     // ---- activation slab staging ---------------------------------------------------------------------------
@@ -209,13 +216,16 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 #pragma unroll
     for (int h = 0; h < 2; ++h) rd_off[h] = ((((8 * h + 2 * lg) ^ li) & 15) << 4);  // piece 8h+2g; its pair is ^16
 
-    auto consume_unit = [&](auto sel, int buf) __attribute__((always_inline)) {
+    // Multiply unit u (register set X, activation buffer `buf`).  The registers of a chunk are free once its tile
+    // is written, so the same chunk of unit u+2 is requested right there, ahead of the LDS reads and the MFMAs.
+    auto consume_unit = [&](auto sel, int buf, bool next_in_range) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
         const uint8_t* const act = act_all + buf * ACT_BYTES;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tb + wr_off[t]) = wq[X][c][t];
+            issue_chunk(sel, c, next_in_range);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -363,13 +373,13 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         constexpr int X = decltype(sel)::value;
         const int ns = next_slab(cs);
         if (u + 1 < u1) act_store(X ^ 1);  // slab of unit u+1, requested one step ago
-        consume_unit(sel, X);
+        act_load(u + 2 < u1);
+        consume_unit(sel, X, u + 2 < u1);
         if (u < u1 && (u + 1 == u1 || ns == 0)) {
             flush_panel(cp, s_first, cs + 1);
             s_first = 0;
         }
-        act_load(u + 2 < u1);
-        issue_unit(sel, u + 2 < u1);
+        issue_done(u + 2 < u1);
         if (u + 1 < u1) __syncthreads();
         cs = ns;
         if (ns == 0) ++cp;
@@ -490,7 +500,7 @@ static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
     if (k % ks != 0 || p->slabs != k / ks || p->panels != (n + bn - 1) / bn) return HFRK_INVALID_CONFIG;
     if (p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
     const long units = (long)p->panels * p->slabs;
-    if (p->grid < 1 || p->grid > kNumCU || p->grid > units) return HFRK_INVALID_CONFIG;
+    if (p->grid < 1 || p->grid > kMaxGrid || p->grid > units) return HFRK_INVALID_CONFIG;
     if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
     return HFRK_SUCCESS;
 }
