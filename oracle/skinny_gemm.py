@@ -47,6 +47,24 @@ def exact_skinny_gemm(skinny_a: torch.Tensor, b: torch.Tensor, scale_a: torch.Te
     return acc
 
 
+def ulp16(ref: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """One unit in the last place of `dtype` (bfloat16 or float16) at |ref|, as float64."""
+    mant, min_exp = (8, -126) if dtype == torch.bfloat16 else (11, -14)
+    e = torch.floor(torch.log2(ref.double().abs().clamp_min(2.0 ** min_exp)))
+    return torch.pow(2.0, e - (mant - 1))
+
+
+def error_bound(skinny_a, b, scale_a, scale_b, dtype: torch.dtype, exact: torch.Tensor) -> torch.Tensor:
+    """Largest |result - exact| an fp32-accumulating implementation with one final rounding may show:
+    one ulp of the 16-bit result (its rounding, with room for a boundary flip) + 2^-16 * sum_k |a_k b_k| scaled
+    (fp32 accumulation in any order over K <= 2^15 terms stays far below this; losing or misplacing a K chunk
+    does not, its effect is of the order of the result)."""
+    abs_a = skinny_a.float().abs().to(torch.float8_e4m3fn)
+    abs_b = b.float().abs().to(torch.float8_e4m3fn)
+    abs_sum = exact_skinny_gemm(abs_a, abs_b, scale_a.abs(), scale_b.abs())
+    return ulp16(exact, dtype) + abs_sum * 2.0 ** -16
+
+
 def int_dot_products(skinny_a: torch.Tensor, b: torch.Tensor) -> np.ndarray:
     """sum_k A[i,k]*B[k,j] as exact integers in units of 2^-18 (int64 [m,n]); slow, for small shapes."""
     ai = np.rint(fp8.decode(skinny_a) * 512.0).astype(np.int64)

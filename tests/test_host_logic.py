@@ -1,0 +1,210 @@
+"""Host-side logic, no GPU: the C ABI loads and exports what the header declares, the launcher's validation
+returns the reference's codes, the planner's decomposition covers every (panel, slab) exactly once and the index
+arithmetic the kernel uses to find a panel's contributors matches brute force, the torch op schemas are the
+reference's, and the Python wrappers reject what the reference's wrappers reject."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from hf_rocm_kernels import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "hfrk_gfx950.h")).read()
+    declared = set(re.findall(r"\b(hfrk_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_capi.SIGNATURES), declared ^ set(_capi.SIGNATURES)
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _capi.load().hfrk_version() >= 100
+    assert _capi.status_string(0) == "success" and "even" in _capi.status_string(2)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_capi, "_lib", None)
+    monkeypatch.setattr(_capi, "LIB_PATH", "/nonexistent/libhfrk_gfx950.so")
+    with pytest.raises(ImportError):
+        _capi.load()
+
+
+def _validate(m=8, n=4096, k=4096, b_stride=None, split_k=1, A=3, B=4, C=3, al=1, bl=4, q=3, op_m=8, ops=4):
+    return _capi.load().hfrk_skinny_gemm_validate(m, n, k, k if b_stride is None else b_stride, split_k, A, B, C, al, bl, q, op_m, ops)
+
+
+def test_validation_codes_match_the_reference_launcher():
+    assert _validate() == _capi.SUCCESS
+    assert _validate(n=4097) == _capi.N_NOT_EVEN
+    assert _validate(k=4096 + 128) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K      # (512/8)*4 = 256
+    assert _validate(k=128, op_m=16, ops=4) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K  # passes the reference's 128, not this kernel's 256
+    assert _validate(A=6, B=6, C=5) == _capi.TOO_MANY_WARPS
+    assert _validate(A=3, B=4, C=3, q=2) == _capi.QSIZE_TOO_SMALL              # consumers > qsize
+    assert _validate(B=8, bl=1, q=3, A=2, C=2) == _capi.QSIZE_TOO_SMALL        # B_producers / b_lanes > qsize
+    assert _validate(op_m=12) == _capi.INVALID_CONFIG
+    assert _validate(ops=2, k=4096) == _capi.INVALID_CONFIG
+    assert _validate(bl=0) == _capi.INVALID_CONFIG
+    # order of the reference's checks: n parity is reported before K divisibility, K before the warp count
+    assert _validate(n=4097, k=100) == _capi.N_NOT_EVEN
+    assert _validate(k=100, A=9, B=9, C=9) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
+    # limits of this implementation
+    assert _validate(m=65) == _capi.BAD_SHAPE
+    assert _validate(b_stride=4096 + 8) == _capi.BAD_ALIGNMENT
+    # every knob set the reference's own table returns is accepted (wrapped.py:45-102 of the reference)
+    for (A, B, C, al, bl, q, om, ops) in [(3, 5, 2, 1, 4, 3, 8, 4), (2, 3, 2, 1, 4, 2, 16, 8), (2, 4, 2, 2, 4, 3, 16, 4),
+                                          (3, 6, 2, 1, 4, 3, 8, 4), (3, 6, 3, 2, 3, 3, 16, 8), (2, 7, 2, 1, 4, 2, 8, 4)]:
+        assert _validate(m=8 if om == 8 else 16, n=16384, k=2048, A=A, B=B, C=C, al=al, bl=bl, q=q, op_m=om, ops=ops) == 0
+
+
+SHAPES = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336), (10240, 8192), (8192, 8192), (57344, 8192),
+          (8192, 28672), (128, 256), (1000, 512), (50, 256), (13312, 16384), (2304, 16384)]
+
+
+def _emulate(plan, n, k):
+    """Replays the kernel's decomposition arithmetic on the host and returns per-panel coverage."""
+    S, P, G = plan.slabs, plan.panels, plan.grid
+    U = S * P
+    ub = lambda g: (g * U) // G
+    cover = [[0] * S for _ in range(P)]
+    contributors = [[] for _ in range(P)]
+    for g in range(G):
+        u0, u1 = ub(g), ub(g + 1)
+        assert u0 < u1, "empty workgroup"
+        for u in range(u0, u1):
+            p, s = divmod(u, S)
+            phys = (s + p % S) % S      # slab rotation: must stay a bijection per panel
+            cover[p][phys] += 1
+            if not contributors[p] or contributors[p][-1] != g:
+                contributors[p].append(g)
+    return cover, contributors, ub
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 33, 64])
+@pytest.mark.parametrize("n,k", SHAPES)
+def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
+    plan = _capi.plan(m, n, k)
+    assert plan.m_tiles == (m + 15) // 16 and plan.wn * plan.wk == 8 and plan.ch in (1, 2)
+    ks = 256 * plan.wk * plan.ch
+    assert k % ks == 0 and plan.slabs == k // ks and plan.panels == -(-n // (16 * plan.wn))
+    assert 1 <= plan.grid <= min(1024, plan.panels * plan.slabs)
+    assert plan.lds_bytes <= 160 * 1024
+    cover, contributors, ub = _emulate(plan, n, k)
+    assert all(c == 1 for row in cover for c in row)
+    S, G, U = plan.slabs, plan.grid, plan.slabs * plan.panels
+    for p, who in enumerate(contributors):
+        lo, hi = p * S, (p + 1) * S
+        g_first = ((lo + 1) * G + U - 1) // U - 1      # the kernel's closed form
+        g_last = (hi * G + U - 1) // U - 1
+        assert who == list(range(g_first, g_last + 1)), (p, who, g_first, g_last)
+        # slot rule: a workgroup's partial for its first panel goes to slot 0, for its last to slot 1; never both the same
+        for g in who:
+            first_panel, last_panel = ub(g) // S, (ub(g + 1) - 1) // S
+            assert p in (first_panel, last_panel) or (ub(g) <= lo and hi <= ub(g + 1))
+
+
+def test_plan_rejects_what_the_kernel_cannot_take():
+    p = _capi.GemmPlan()
+    lib = _capi.load()
+    assert lib.hfrk_skinny_gemm_plan(65, 128, 256, ctypes.byref(p)) == _capi.BAD_SHAPE
+    assert lib.hfrk_skinny_gemm_plan(0, 128, 256, ctypes.byref(p)) == _capi.BAD_SHAPE
+    assert lib.hfrk_skinny_gemm_plan(8, 128, 300, ctypes.byref(p)) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
+    assert lib.hfrk_skinny_gemm_plan(8, 128, 256, None) == _capi.BAD_SHAPE
+
+
+def test_op_schemas_are_the_reference_schemas():
+    import hf_rocm_kernels  # noqa: F401  (loads _HFRK_C)
+    # the definition strings of the reference's csrc/torch_bindings.cpp:22,26-28,32-34,38-40, verbatim
+    expect = {
+        "increment": "increment(Tensor! x) -> ()",
+        "residual_rms": "residual_rms(Tensor input, Tensor! residual, Tensor weight, Tensor scale_tensor, float epsilon, Tensor! "
+                        "output, Tensor! next_buffer, int num_threads, bool force_scalar) -> ()",
+        "swiglu": "swiglu(Tensor gate_up, Tensor scale_tensor, Tensor! output, Tensor! next_buffer, int num_threads, "
+                  "bool force_scalar) -> ()",
+        "skinny_gemm_tb": "skinny_gemm_tb(Tensor A, Tensor B, Tensor! D, Tensor scale_tensor, int split_k, int A_producers, "
+                          "int B_producers, int consumers, int a_lanes, int b_lanes, int qsize, int op_m, int ops) -> int",
+    }
+    for name, schema in expect.items():
+        got = getattr(torch.ops._HFRK_C, name).default._schema
+        want = torch._C.parse_schema("_HFRK_C::" + schema)
+        assert str(got) == str(want), (str(got), str(want))
+        assert [(a.name, str(a.type), a.alias_info is not None and a.alias_info.is_write) for a in got.arguments] == \
+               [(a.name, str(a.type), a.alias_info is not None and a.alias_info.is_write) for a in want.arguments]
+
+
+def test_ops_have_no_cpu_path():
+    import hf_rocm_kernels  # noqa: F401
+    a = torch.zeros(8, 256).to(torch.float8_e4m3fn)
+    b = torch.zeros(128, 256).to(torch.float8_e4m3fn).t()
+    d = torch.zeros(8, 128, dtype=torch.bfloat16)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops._HFRK_C.skinny_gemm_tb(a, b, d, torch.ones(1), 1, 3, 4, 3, 1, 4, 3, 8, 4)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops._HFRK_C.swiglu(torch.zeros(2, 16, dtype=torch.float16), torch.ones(1), torch.zeros(2, 8).to(torch.float8_e4m3fn),
+                                 torch.zeros(2, 0, dtype=torch.float16), 64, False)
+
+
+def test_wrapper_assertions_mirror_the_reference():
+    from hf_rocm_kernels import residual_rms, skinny_gemm, swiglu
+    from hf_rocm_kernels.operators.residual_rms.wrapped import infer_num_threads as rms_threads
+    from hf_rocm_kernels.operators.skinny_gemm.wrapped import infer_skinny_gemm_m_params, skinny_gemm_checks
+    from hf_rocm_kernels.operators.swiglu.wrapped import infer_num_threads as swiglu_threads
+
+    a = torch.zeros(8, 256).to(torch.float8_e4m3fn)
+    b = torch.zeros(128, 256).to(torch.float8_e4m3fn).t()
+    d = torch.zeros(8, 128, dtype=torch.bfloat16)
+    one = torch.ones(1)
+    with pytest.raises(AssertionError, match="cuda"):     # device check comes last, as in the reference
+        skinny_gemm(a, b, one, d)
+    with pytest.raises(AssertionError, match="2 dimensions"):
+        skinny_gemm_checks(a[0], b, one, d)
+    with pytest.raises(AssertionError, match="to be the same"):
+        skinny_gemm_checks(a[:, :128].contiguous(), b, one, d)
+    with pytest.raises(AssertionError, match="to be 1"):
+        skinny_gemm_checks(a, b, torch.ones(2), d)
+    with pytest.raises(AssertionError, match="column-major"):
+        skinny_gemm_checks(a, b.t().contiguous().t().contiguous(), one, d)
+    with pytest.raises(AssertionError, match="float8_e4m3fn"):
+        skinny_gemm_checks(a.view(torch.uint8).view(torch.float8_e4m3fnuz), b, one, d)
+    with pytest.raises(AssertionError, match="bfloat16 or torch.float16"):
+        skinny_gemm_checks(a, b, one, d.float())
+    assert infer_skinny_gemm_m_params(8) == (1, 8) and infer_skinny_gemm_m_params(16) == (1, 16)
+    assert infer_skinny_gemm_m_params(17) == (2, 16)
+    x = torch.zeros(4, 64, dtype=torch.float16)
+    with pytest.raises(AssertionError, match="cuda"):
+        residual_rms(x, x.clone(), torch.ones(64, dtype=torch.float16), 1e-5)
+    with pytest.raises(AssertionError, match="same shape"):
+        residual_rms(x, x[:2].clone(), torch.ones(64, dtype=torch.float16), 1e-5)
+    with pytest.raises(ValueError):
+        rms_threads(4, 2048)
+    assert rms_threads(4, 0) == 0 and rms_threads(4, 100) == 128 and rms_threads(4, 1024) == 1024
+    with pytest.raises(AssertionError, match="even number of columns"):
+        swiglu(torch.zeros(4, 63, dtype=torch.float16), one)
+    with pytest.raises(AssertionError, match="cuda"):
+        swiglu(torch.zeros(4, 64, dtype=torch.float16), one)
+    assert swiglu_threads(8, False, 128) == 128 and swiglu_threads(8, False, -1) == 256
+
+
+def test_data_generators_are_seeded_and_follow_the_recipes():
+    from hf_rocm_kernels.operators.residual_rms import generate_residual_rms_data
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data, generate_skinny_gemm_data
+    from hf_rocm_kernels.operators.swiglu import generate_swiglu_data
+    from oracle import skinny_gemm as og
+
+    a, b, s, out = generate_skinny_gemm_data(4, 32, 256, seed=0, device="cpu")
+    a2, b2, s2, _ = generate_skinny_gemm_data(4, 32, 256, seed=0, device="cpu")
+    oa, ob, os_, _ = og.generate_skinny_gemm_data(4, 32, 256, seed=0)   # the oracle's twin draws the same bits
+    for x, y, z in ((a, a2, oa), (b, b2, ob)):
+        assert torch.equal(x.view(torch.uint8), y.view(torch.uint8)) and torch.equal(x.view(torch.uint8), z.view(torch.uint8))
+    assert torch.equal(s, s2) and torch.equal(s, os_) and 1 <= float(s) < 3
+    assert a.shape == (4, 256) and b.shape == (256, 32) and b.stride(0) == 1 and out.shape == (4, 32) and out.abs().sum() == 0
+    a, w, sa, sw = generate_llama_gemm_data(16, 64, 512, seed=1, device="cpu", per_token=True, per_channel=True, outlier_rows=(3,))
+    assert sa.shape == (16,) and sw.shape == (64,) and w.stride(0) == 1
+    assert float(sa[3]) > 5 * float(sa.median())          # the x20 outlier row gets its own, larger scale
+    assert (a.float().abs().amax(dim=1) == 448).all()
+    x, r, wt, eps, sc, nb = generate_residual_rms_data(3, 64, 16, dtype=torch.float8_e4m3fn, seed=2, device="cpu", io_dtype=torch.bfloat16)
+    assert x.dtype == torch.bfloat16 and sc is not None and nb.shape == (3, 16) and 1e-5 <= eps < 2e-5
+    gu, sc, nb = generate_swiglu_data(3, 32, 0, seed=3, device="cpu")
+    assert gu.shape == (3, 64) and nb is None
