@@ -23,7 +23,7 @@ OBJ = os.path.join(HERE, "build")
 INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["hfrk_common.hip", "skinny_gemm.hip", "residual_rms.hip", "swiglu.hip"]
+HIP_SOURCES = ["hfrk_common.hip", "skinny_gemm.hip", "skinny_gemm_stream.hip", "residual_rms.hip", "swiglu.hip"]
 LIB_NAME = "libhfrk_gfx950.so"
 EXT_NAME = "_HFRK_C.abi3.so"
 
@@ -95,7 +95,7 @@ def _link_torch_extension(obj):
 def build_all(with_torch=True):
     """Compile everything, every time it is called: objects in parallel, then the two links."""
     os.makedirs(OBJ, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=5) as pool:
+    with ThreadPoolExecutor(max_workers=6) as pool:
         hip_jobs = [pool.submit(_compile_hip, s) for s in HIP_SOURCES]
         ext_job = pool.submit(_compile_torch_bindings) if with_torch else None
         objs = [j.result() for j in hip_jobs]

@@ -26,31 +26,9 @@
 #include <mutex>
 #include <type_traits>
 
-#include "hfrk_internal.h"
+#include "skinny_gemm_args.h"
 
 namespace hfrk {
-
-constexpr int kGemmWaves = 8;
-constexpr int kGemmThreads = kGemmWaves * kWave;
-constexpr int kTileBytes = 4096;                 // 16 rows x 256 B, one chunk of one wave
-constexpr int kLdsLimit = 160 * 1024;            // LDS per CU on gfx950
-constexpr int kMaxPanels = 1 << 20;              // per-panel arrival counters
-constexpr int kMaxGrid = 4 * kNumCU;              // persistent workgroups: up to 4 per CU when LDS and registers allow
-constexpr size_t kWsFloats = (size_t)2 * kMaxGrid * kGemmWaves * 4 * 256;  // 2 slots x grid x WN*MT KB (worst case)
-
-struct GemmArgs {
-    const uint8_t* A;
-    const uint8_t* B;
-    void* D;
-    const float* scale_a;
-    const float* scale_b;
-    int sa_stride, sb_stride;
-    int m, n, k, b_stride;
-    int d_dtype, accumulate;
-    int panels, slabs, units, grid, nbuf;
-    float* ws;
-    int* counters;
-};
 
 // first unit of logical workgroup g
 __device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (int)(((long)g * units) / grid); }
@@ -457,9 +435,29 @@ static double plan_cost(int n, int k, int mt, int wn, int wk, int ch, int* grid_
     return (stream + upw * per_unit + flush + fixup) * (1.0 + waste);
 }
 
+// m <= 16: every wave streams its own run of (16-row tile, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
+static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    const long tiles = (n + 15) / 16;
+    if (tiles > kMaxPanels) return HFRK_BAD_SHAPE;
+    const int kc = k / 256;
+    const long chunks = tiles * kc;
+    long grid = chunks < kNumCU ? chunks : kNumCU;
+    if (grid >= 8) grid -= grid % 8;  // whole XCD groups
+    plan->m_tiles = 1;
+    plan->wn = 0;
+    plan->wk = 0;
+    plan->ch = (m + 3) / 4;
+    plan->grid = (int)grid;
+    plan->panels = (int)tiles;
+    plan->slabs = kc;
+    plan->lds_bytes = kStreamLdsBytes;
+    return HFRK_SUCCESS;
+}
+
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (m <= 16) return make_stream_plan(m, n, k, plan);
     const int mt = (m + 15) / 16;
     static const int wns[4] = {1, 2, 4, 8};
     double best = 1e300;
@@ -493,6 +491,14 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 }
 
 static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
+    if (p->wn == 0) {  // wave-stream decomposition
+        if (m > 16 || p->m_tiles != 1 || p->wk != 0 || p->ch < 1 || p->ch > 4 || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
+        if (p->panels != (n + 15) / 16 || p->slabs != k / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
+        const long chunks = (long)p->panels * p->slabs;
+        if (p->grid < 1 || p->grid > kMaxGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
+        if (p->lds_bytes != kStreamLdsBytes) return HFRK_INVALID_CONFIG;
+        return HFRK_SUCCESS;
+    }
     if (p->m_tiles < 1 || p->m_tiles > 4 || p->m_tiles * 16 < m) return HFRK_INVALID_CONFIG;
     if (!(p->wn == 1 || p->wn == 2 || p->wn == 4 || p->wn == 8) || p->wn * p->wk != kGemmWaves) return HFRK_INVALID_CONFIG;
     if (p->ch != 1 && p->ch != 2) return HFRK_INVALID_CONFIG;
@@ -588,6 +594,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const float* scale
         // D rows would be misaligned for 8-byte stores: report rather than take a slow path silently
         return HFRK_BAD_ALIGNMENT;
     }
+    if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.lds_bytes, stream);
     switch (p.m_tiles) {
         case 1: return launch_mt<1>(args, p, stream);
         case 2: return launch_mt<2>(args, p, stream);

@@ -1,0 +1,260 @@
+// FP8 skinny GEMM, m <= 16: every wavefront streams its own run of weight chunks, nothing else is shared.
+//
+// The weight matrix is cut into chunks of 16 rows x 256 K-bytes (4 KB), numbered row tile by row tile, K fastest.
+// The chunk sequence is split evenly over the workgroups and, inside a workgroup, evenly over its 8 waves, so a
+// wave owns one contiguous run: part of a row tile, then whole row tiles, then part of another.  For each chunk
+// the wave loads the 4 KB of weights (four 16-byte `nt` loads per lane, 4 rows x 256 contiguous bytes per
+// instruction) and the matching m x 256 bytes of activations (L1/L2 hits; rows >= m are out of range and cost
+// nothing), turns both into MFMA operand layout through two private, XOR-swizzled LDS tiles, and issues two
+// v_mfma_f32_16x16x128_f8f6f4.  The next chunk's loads are issued as soon as the registers have been copied to
+// LDS.  There is no barrier, no shared staging and no cross-wave dependency in the loop: measured, this loop
+// sustains the same bandwidth as a kernel that only reads the weights.
+//
+// Sums that a wave cannot finish alone (a row tile split between waves) are combined once, after the loop:
+// partial 16x16 fp32 tiles go to LDS, one barrier, and the wave that holds a tile's first K chunk adds the others
+// in wave order.  A row tile split between workgroups goes through the workspace with a per-tile arrival counter;
+// the last workgroup to arrive adds the partials in workgroup order.  Both orders are fixed, so results are
+// bit-reproducible.  Scales, the optional accumulate-into-D and the single rounding to 16 bits happen there.
+//
+// Replaces, for m <= 16, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and
+// consumers (producers/n_full_tiles.cu:4-127, consumers/mfma_16x16x32_consumer.cu:1-168,
+// consumers/smfma_16x16x64_consumer.cu:1-158).
+#include "skinny_gemm_args.h"
+
+namespace hfrk {
+
+// MA = 16-byte activation loads per lane and chunk: load t brings rows 4t .. 4t+3, so 4*MA >= m.
+template <int MA>
+__global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const GemmArgs a) {
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    constexpr int kCoherent = 17;  // sc0 | sc1
+
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t* const tiles = lds;                                                 // per wave: weight tile, activation tile
+    v4f* const slots = reinterpret_cast<v4f*>(lds + kGemmWaves * 2 * kTileBytes);  // [wave][2][64 lanes]
+    int* const meta = reinterpret_cast<int*>(lds + kGemmWaves * 2 * kTileBytes + kGemmWaves * 2 * 1024);  // [wave][2][tile,kb,ke,_]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+
+    const int G = a.grid;
+    const int KC = a.slabs;                      // 256-byte chunks per row tile
+    const long C = (long)a.panels * KC;          // all chunks
+    const int b = blockIdx.x;
+    const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;  // XCD x owns logical ids [x*G/8, (x+1)*G/8)
+    const long c0 = g * C / G, c1 = (g + 1) * C / G;
+    const long nwg = c1 - c0;
+    const long w0 = c0 + wv * nwg / kGemmWaves, w1 = c0 + (wv + 1) * nwg / kGemmWaves;
+    const int count = (int)(w1 - w0);
+
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
+    uint16_t* const D = reinterpret_cast<uint16_t*>(a.D);
+
+    const int mrow = li;  // the activation row (= output row) this lane's accumulator column belongs to
+    const float sa = a.scale_a[(long)min(mrow, a.m - 1) * a.sa_stride] *
+                     ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+
+    // ---- streaming loop ---------------------------------------------------------------------------------------
+    const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
+    const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
+    uint8_t* const tw = tiles + wv * 2 * kTileBytes;
+    uint8_t* const ta = tw + kTileBytes;
+    int wr_off[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int row = 4 * t + lg;
+        wr_off[t] = row * 256 + ((li ^ row) << 4);
+    }
+    int rd_off[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) rd_off[h] = li * 256 + ((((8 * h + 2 * lg) ^ li) & 15) << 4);
+
+    v4i wq[4], aq[MA];
+    int tile = (int)(w0 / KC), kc = (int)(w0 % KC);  // chunk being multiplied
+    int itile = tile, ikc = kc;                      // chunk being requested
+    auto issue = [&](bool in_range) __attribute__((always_inline)) {
+        const uint32_t abase = in_range ? (uint32_t)ikc * 256u : kOutOfRange;
+        const uint32_t wbase = in_range ? (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)ikc * 256u : kOutOfRange;
+#pragma unroll
+        for (int t = 0; t < MA; ++t)
+            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+        if (++ikc == KC) { ikc = 0; ++itile; }
+    };
+
+    // scale, add D (accumulate mode), round once, store: lane holds D^T[n0 + v][mrow], v = 0..3
+    auto epilogue = [&](int t, v4f acc) __attribute__((always_inline)) {
+        const int n0 = t * 16 + 4 * lg;
+        if (mrow >= a.m || n0 >= a.n) return;
+        uint16_t* const drow = D + (long)mrow * a.n;
+        const bool vec = ((a.n & 3) == 0);  // then n0 + 3 < n and the 8-byte access is aligned
+        uint32_t old[4] = {0u, 0u, 0u, 0u};
+        float sb[4] = {1.f, 1.f, 1.f, 1.f};
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int n = min(n0 + v, a.n - 1);
+            if (a.scale_b && a.sb_stride) sb[v] = a.scale_b[n];
+        }
+        if (a.accumulate) {
+            if (vec) {
+                const uint2 q = *reinterpret_cast<const uint2*>(drow + n0);
+                old[0] = q.x & 0xffffu; old[1] = q.x >> 16; old[2] = q.y & 0xffffu; old[3] = q.y >> 16;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) old[v] = drow[min(n0 + v, a.n - 1)];
+            }
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float r = acc[v] * (sa * sb[v]);
+            const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)old[v]) : load16<HFRK_F16>((uint16_t)old[v]);
+            const float sum = a.accumulate ? base + r : r;
+            o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
+        }
+        if (vec) {
+            *reinterpret_cast<uint2*>(drow + n0) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n0 + v < a.n) drow[n0 + v] = (uint16_t)o[v];
+        }
+    };
+
+    // A wave's run is: [head segment] [whole row tiles ...] [last segment]; head/last may be partial tiles.
+    const int tile_h = tile, kb_h = kc;
+    const int ke_h = (int)min((long)KC, (long)kb_h + count);
+    const bool head_partial = count > 0 && !(kb_h == 0 && ke_h == KC);
+    const int tile_l = count > 0 ? (int)((w1 - 1) / KC) : -1;
+    const int ke_l = count > 0 ? (int)((w1 - 1) % KC) + 1 : 0;
+    const bool last_distinct = count > 0 && tile_l != tile_h;
+    const bool last_partial = last_distinct && ke_l != KC;
+
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    v4f part_h = {0.f, 0.f, 0.f, 0.f};
+
+    issue(count > 0);
+    for (int i = 0; i < count; ++i) {
+#pragma unroll
+        for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + wr_off[t]) = wq[t];
+        issue(i + 1 < count);  // registers are free again: request the next chunk before the LDS reads and MFMAs
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const v4i wlo = *reinterpret_cast<const v4i*>(tw + rd_off[h]);
+            const v4i whi = *reinterpret_cast<const v4i*>(tw + (rd_off[h] ^ 16));
+            const v4i alo = *reinterpret_cast<const v4i*>(ta + rd_off[h]);
+            const v4i ahi = *reinterpret_cast<const v4i*>(ta + (rd_off[h] ^ 16));
+            const v8i wop = {wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
+            const v8i aop = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc, 0, 0, 0, 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (++kc == KC) {  // a row tile ends inside this wave's run
+            if (tile == tile_h && head_partial) part_h = acc;   // its first chunks belong to an earlier wave
+            else epilogue(tile, acc);                           // all of it was ours
+            acc = v4f{0.f, 0.f, 0.f, 0.f};
+            kc = 0;
+            ++tile;
+        }
+    }
+    // here: acc = sums of the last segment if it is partial (else zero); part_h = head segment if it ended a tile.
+    // A run that lies inside one tile and does not end it leaves its only segment in acc: treat it as the head.
+    const bool single = count > 0 && !last_distinct;
+    if (single && head_partial && ke_h != KC) part_h = acc;
+
+    // ---- combine the partial tiles of this workgroup ------------------------------------------------------------
+    // slot 0: head segment, slot 1: last segment (when it is another tile).  meta: tile (-1 = none), kb, ke.
+    {
+        int* const mine = meta + wv * 8;
+        if (lane == 0) {
+            mine[0] = head_partial ? tile_h : -1; mine[1] = kb_h; mine[2] = ke_h;
+            mine[4] = last_partial ? tile_l : -1; mine[5] = 0;    mine[6] = ke_l;
+        }
+        if (head_partial) slots[(wv * 2 + 0) * 64 + lane] = part_h;
+        if (last_partial) slots[(wv * 2 + 1) * 64 + lane] = acc;
+    }
+    __syncthreads();
+
+    // A segment that starts its tile inside this workgroup (first K chunk of the tile, or first chunk of the
+    // workgroup's range) makes this wave the one that finishes the tile: add the following waves' head segments.
+    auto finish_segment = [&](int t, int kb, int ke, v4f sum) __attribute__((always_inline)) {
+        for (int j = wv + 1; j < kGemmWaves && ke < KC; ++j) {
+            const int* const mj = meta + j * 8;
+            if (mj[0] != t) {
+                if (mj[0] == -1 && mj[4] == -1 && mj[2] == mj[1]) continue;  // a wave without chunks
+                break;
+            }
+            sum += slots[(j * 2 + 0) * 64 + lane];
+            ke = mj[2];
+        }
+        if (kb == 0 && ke == KC) {
+            epilogue(t, sum);
+            return;
+        }
+        // the tile continues in a neighbouring workgroup: park this workgroup's share, count the arrival
+        const int slot = (t == (int)(c0 / KC)) ? 0 : 1;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum), ws_rsrc, ((g * 2 + slot) * 64 + lane) * 16, 0, kCoherent);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's store acknowledged before the arrival is counted
+        int last = 0;
+        if (lane == 0) {
+            const int mine = ke - kb;
+            const int seen = atomicAdd(&a.counters[t], mine);
+            last = (seen + mine == KC);
+            if (last) a.counters[t] = 0;  // ready for the next launch
+        }
+        last = __builtin_amdgcn_readfirstlane(last);
+        if (!last) return;
+        const long lo = (long)t * KC, hi = lo + KC;
+        const int g_first = (int)(((lo + 1) * G + C - 1) / C) - 1;
+        const int g_last = (int)((hi * G + C - 1) / C) - 1;
+        v4f total = {0.f, 0.f, 0.f, 0.f};
+        for (int gg = g_first; gg <= g_last; ++gg) {
+            const int sl = ((int)((gg * C / G) / KC) == t) ? 0 : 1;
+            total += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ((gg * 2 + sl) * 64 + lane) * 16, 0, kCoherent));
+        }
+        epilogue(t, total);
+    };
+    if (head_partial && (kb_h == 0 || w0 == c0)) finish_segment(tile_h, kb_h, ke_h, part_h);
+    if (last_partial) finish_segment(tile_l, 0, ke_l, acc);
+}
+
+int launch_stream_kernel(const GemmArgs& args, int act_loads, int lds_bytes, hipStream_t stream) {
+#define HFRK_STREAM_CASE(MA_)                                                                                       \
+    case MA_: {                                                                                                     \
+        auto kern = skinny_gemm_stream_kernel<MA_>;                                                                 \
+        static bool attr_done[64] = {};                                                                             \
+        int dev = 0;                                                                                                \
+        HFRK_HIP_TRY(hipGetDevice(&dev));                                                                           \
+        if (dev >= 0 && dev < 64 && !attr_done[dev]) {                                                              \
+            HFRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                   \
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));               \
+            attr_done[dev] = true;                                                                                  \
+        }                                                                                                           \
+        hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);                     \
+        break;                                                                                                      \
+    }
+    switch (act_loads) {
+        HFRK_STREAM_CASE(1)
+        HFRK_STREAM_CASE(2)
+        HFRK_STREAM_CASE(3)
+        HFRK_STREAM_CASE(4)
+        default: return HFRK_INVALID_CONFIG;
+    }
+#undef HFRK_STREAM_CASE
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}
+
+}  // namespace hfrk

@@ -48,12 +48,14 @@ enum hfrk_dtype { HFRK_F16 = 0, HFRK_BF16 = 1, HFRK_FP8_E4M3FN = 2 };
  * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102 and benchmarks/skinny_gemm/grid_search.py). */
 typedef struct hfrk_gemm_plan {
     int m_tiles;   /* ceil(m/16): 16-row activation tiles kept in registers (1..4) */
-    int wn;        /* waves of a workgroup spread over output rows (16 weight rows each) */
-    int wk;        /* waves of a workgroup spread over K; wn*wk = 8 waves */
-    int ch;        /* 256-byte K chunks each wave streams per slab (1 or 2) */
-    int grid;      /* persistent workgroups launched (<= 256, one per CU) */
-    int panels;    /* ceil(n / (16*wn)) */
-    int slabs;     /* k / (256*wk*ch): K slabs per panel */
+    int wn;        /* 0: wave-stream decomposition (m <= 16), every wave streams its own run of chunks.
+                      1,2,4,8: workgroup decomposition, wn waves spread over output rows (16 weight rows each) */
+    int wk;        /* workgroup decomposition: waves spread over K, wn*wk = 8.  wave-stream: 0 */
+    int ch;        /* workgroup decomposition: 256-byte K chunks each wave streams per slab (1 or 2).
+                      wave-stream: 16-byte activation loads per lane and chunk, ceil(m/4) */
+    int grid;      /* persistent workgroups launched */
+    int panels;    /* workgroup decomposition: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n/16) row tiles */
+    int slabs;     /* workgroup decomposition: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per tile */
     int lds_bytes; /* dynamic LDS per workgroup */
 } hfrk_gemm_plan;
 

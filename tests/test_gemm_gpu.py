@@ -57,6 +57,10 @@ def all_plans(m, n, k):
     from hf_rocm_kernels import _capi
     mt = (m + 15) // 16
     plans = []
+    if m <= 16:  # wave-stream decomposition: grids that split row tiles between workgroups in different ways
+        tiles, kc = (n + 15) // 16, k // 256
+        for grid in sorted({min(256, tiles * kc), min(200, tiles * kc), min(7, tiles * kc), min(512, tiles * kc), 1}):
+            plans.append(_capi.GemmPlan(1, 0, 0, (m + 3) // 4, grid, tiles, kc, 8 * 2 * 4096 + 8 * 2 * 1024 + 256))
     for wn in (1, 2, 4, 8):
         wk = 8 // wn
         for ch in (1, 2):
@@ -85,7 +89,8 @@ def test_default_plan_matches_oracle(m, n, k):
     check_against_oracle(out, a, b, sa, sw)
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336)])
+@pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
+                                   (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024)])
 def test_every_plan_gives_the_same_answer(m, n, k):
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=7)

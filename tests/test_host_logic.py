@@ -63,6 +63,24 @@ SHAPES = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336), (10240, 8192
           (8192, 28672), (128, 256), (1000, 512), (50, 256), (13312, 16384), (2304, 16384)]
 
 
+def _emulate_stream(plan):
+    """Wave-stream decomposition: chunks (row tile, K chunk) split over workgroups, then over their 8 waves."""
+    KC, T, G = plan.slabs, plan.panels, plan.grid
+    C = T * KC
+    cover = [0] * C
+    wg_of_tile = [[] for _ in range(T)]
+    for g in range(G):
+        c0, c1 = g * C // G, (g + 1) * C // G
+        assert c0 < c1
+        n = c1 - c0
+        for w in range(8):
+            for c in range(c0 + w * n // 8, c0 + (w + 1) * n // 8):
+                cover[c] += 1
+        for t in range(c0 // KC, (c1 - 1) // KC + 1):
+            wg_of_tile[t].append(g)
+    return cover, wg_of_tile
+
+
 def _emulate(plan, n, k):
     """Replays the kernel's decomposition arithmetic on the host and returns per-panel coverage."""
     S, P, G = plan.slabs, plan.panels, plan.grid
@@ -86,6 +104,17 @@ def _emulate(plan, n, k):
 @pytest.mark.parametrize("n,k", SHAPES)
 def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
     plan = _capi.plan(m, n, k)
+    if plan.wn == 0:  # m <= 16: wave-stream decomposition
+        assert m <= 16 and plan.ch == (m + 3) // 4 and plan.panels == -(-n // 16) and plan.slabs == k // 256
+        assert 1 <= plan.grid <= min(256, plan.panels * plan.slabs) and plan.lds_bytes <= 160 * 1024
+        cover, wg_of_tile = _emulate_stream(plan)
+        assert all(c == 1 for c in cover)
+        KC, G, C = plan.slabs, plan.grid, plan.panels * plan.slabs
+        for t, who in enumerate(wg_of_tile):
+            lo, hi = t * KC, (t + 1) * KC
+            assert who == list(range(((lo + 1) * G + C - 1) // C - 1, (hi * G + C - 1) // C)), (t, who)
+        return
+    assert m > 16
     assert plan.m_tiles == (m + 15) // 16 and plan.wn * plan.wk == 8 and plan.ch in (1, 2)
     ks = 256 * plan.wk * plan.ch
     assert k % ks == 0 and plan.slabs == k // ks and plan.panels == -(-n // (16 * plan.wn))
