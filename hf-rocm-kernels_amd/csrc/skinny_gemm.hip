@@ -31,7 +31,8 @@
 namespace hfrk {
 
 // first unit of logical workgroup g
-__device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (int)(((long)g * units) / grid); }
+// 32-bit on purpose (64-bit division is a long instruction sequence); the host checks units * (grid + 1) < 2^31.
+__device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (int)(((uint32_t)g * (uint32_t)units) / (uint32_t)grid); }
 
 template <int MT, int WN, int WK, int CH>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArgs a) {
@@ -310,9 +311,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             const int last = *flag;
             if (last && wk == 0) {
                 // contributors are the workgroups whose unit range meets [panel*S, (panel+1)*S), in id order
-                const long lo = (long)panel * S, hi = lo + S;
-                const int g_first = (int)(((lo + 1) * G + U - 1) / U) - 1;
-                const int g_last = (int)((hi * G + U - 1) / U) - 1;
+                const uint32_t lo = (uint32_t)panel * (uint32_t)S, hi = lo + (uint32_t)S;
+                const int g_first = (int)(((lo + 1) * (uint32_t)G + (uint32_t)U - 1) / (uint32_t)U) - 1;
+                const int g_last = (int)((hi * (uint32_t)G + (uint32_t)U - 1) / (uint32_t)U) - 1;
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
                 for (int gg = g_first; gg <= g_last; ++gg) {
@@ -496,6 +497,7 @@ static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
         if (p->panels != (n + 15) / 16 || p->slabs != k / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
         const long chunks = (long)p->panels * p->slabs;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
+        if (chunks * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's chunk arithmetic is 32-bit
         if (p->lds_bytes != kStreamLdsBytes) return HFRK_INVALID_CONFIG;
         return HFRK_SUCCESS;
     }
@@ -507,6 +509,7 @@ static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
     if (p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
     const long units = (long)p->panels * p->slabs;
     if (p->grid < 1 || p->grid > kMaxGrid || p->grid > units) return HFRK_INVALID_CONFIG;
+    if (units * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's unit arithmetic is 32-bit
     if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
     return HFRK_SUCCESS;
 }

@@ -29,6 +29,6 @@ struct GemmArgs {
 
 // wave-stream kernel (m <= 16), skinny_gemm_stream.hip
 int launch_stream_kernel(const GemmArgs& args, int act_loads, int lds_bytes, hipStream_t stream);
-constexpr int kStreamLdsBytes = kGemmWaves * 2 * kTileBytes + kGemmWaves * 2 * 1024 + 256;
+constexpr int kStreamLdsBytes = kGemmWaves * 2 * kTileBytes + 256;
 
 }  // namespace hfrk

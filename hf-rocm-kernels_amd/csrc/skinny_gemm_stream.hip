@@ -30,9 +30,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     constexpr int kCoherent = 17;  // sc0 | sc1
 
     extern __shared__ __align__(16) uint8_t lds[];
-    uint8_t* const tiles = lds;                                                 // per wave: weight tile, activation tile
-    v4f* const slots = reinterpret_cast<v4f*>(lds + kGemmWaves * 2 * kTileBytes);  // [wave][2][64 lanes]
-    int* const meta = reinterpret_cast<int*>(lds + kGemmWaves * 2 * kTileBytes + kGemmWaves * 2 * 1024);  // [wave][2][tile,kb,ke,_]
+    uint8_t* const tiles = lds;  // per wave: weight tile, activation tile
+    // After its loop a wave's tiles are dead; its two partial-sum slots (64 lanes x 16 bytes each) reuse the start of
+    // its own weight tile, so no other wave's data is touched before the barrier.
+    v4f* const slots = reinterpret_cast<v4f*>(lds);  // slot s of wave w at byte w*2*kTileBytes + s*1024
+    constexpr int kSlotStride = 2 * kTileBytes / 16;  // in v4f
+    int* const meta = reinterpret_cast<int*>(lds + kGemmWaves * 2 * kTileBytes);  // [wave][2][tile,kb,ke,_]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -41,22 +44,25 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 
     const int G = a.grid;
     const int KC = a.slabs;                      // 256-byte chunks per row tile
-    const long C = (long)a.panels * KC;          // all chunks
+    // All chunk arithmetic fits 32 bits: the host checks grid * chunks < 2^31 (64-bit division costs microseconds here).
+    const uint32_t C = (uint32_t)a.panels * (uint32_t)KC;  // all chunks
     const int b = blockIdx.x;
     const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;  // XCD x owns logical ids [x*G/8, (x+1)*G/8)
-    const long c0 = g * C / G, c1 = (g + 1) * C / G;
-    const long nwg = c1 - c0;
-    const long w0 = c0 + wv * nwg / kGemmWaves, w1 = c0 + (wv + 1) * nwg / kGemmWaves;
+    const uint32_t c0 = (uint32_t)g * C / (uint32_t)G, c1 = (uint32_t)(g + 1) * C / (uint32_t)G;
+    const uint32_t nwg = c1 - c0;
+    const uint32_t w0 = c0 + (uint32_t)wv * nwg / kGemmWaves, w1 = c0 + (uint32_t)(wv + 1) * nwg / kGemmWaves;
     const int count = (int)(w1 - w0);
 
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
-    uint16_t* const D = reinterpret_cast<uint16_t*>(a.D);
+    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
+    const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
+    const bool vec = ((a.n & 3) == 0);  // then a lane's four outputs n0 .. n0+3 are all inside n and 8-byte aligned
+    const bool per_channel = a.scale_b && a.sb_stride;
 
     const int mrow = li;  // the activation row (= output row) this lane's accumulator column belongs to
-    const float sa = a.scale_a[(long)min(mrow, a.m - 1) * a.sa_stride] *
-                     ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+    float sa = 1.0f;      // scale_a[row] * (scalar scale_b), loaded once the stream is under way
 
     // ---- streaming loop ---------------------------------------------------------------------------------------
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
@@ -73,8 +79,21 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 #pragma unroll
     for (int h = 0; h < 2; ++h) rd_off[h] = li * 256 + ((((8 * h + 2 * lg) ^ li) & 15) << 4);
 
+    // Old D values (accumulate mode) and per-channel scales of one row tile, requested ahead of the epilogue that
+    // uses them.  Only for the aligned case; out-of-range offsets make the loads free where they are not wanted.
+    struct Pre { v2i d; v4i sb; };
+    auto prefetch = [&](int t, bool wanted) __attribute__((always_inline)) {
+        const int n0 = t * 16 + 4 * lg;
+        const bool ok = wanted && vec && li < a.m && n0 < a.n;
+        Pre p;
+        p.d = __builtin_amdgcn_raw_buffer_load_b64(d_rsrc, (ok && a.accumulate) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
+        p.sb = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (ok && per_channel) ? n0 * 4 : (int)kOutOfRange, 0, 0);
+        return p;
+    };
+    Pre pre_next, pre_cur;
     v4i wq[4], aq[MA];
-    int tile = (int)(w0 / KC), kc = (int)(w0 % KC);  // chunk being multiplied
+    int tile = (int)(w0 / (uint32_t)KC);             // chunk being multiplied
+    int kc = (int)(w0 - (uint32_t)tile * (uint32_t)KC);
     int itile = tile, ikc = kc;                      // chunk being requested
     auto issue = [&](bool in_range) __attribute__((always_inline)) {
         const uint32_t abase = in_range ? (uint32_t)ikc * 256u : kOutOfRange;
@@ -85,54 +104,55 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 #pragma unroll
         for (int t = 0; t < 4; ++t)
             wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+        pre_next = prefetch(itile, in_range && ikc == KC - 1);  // the chunk that ends a row tile brings the tile's D along
         if (++ikc == KC) { ikc = 0; ++itile; }
     };
 
-    // scale, add D (accumulate mode), round once, store: lane holds D^T[n0 + v][mrow], v = 0..3
-    auto epilogue = [&](int t, v4f acc) __attribute__((always_inline)) {
+    // scale, add D (accumulate mode), round once, store: lane holds D^T[n0 + v][mrow], v = 0..3.
+    // Aligned n: D and the channel scales were prefetched (pre), one 8-byte store.  Ragged n (n % 4 != 0): 2-byte
+    // buffer accesses whose out-of-range offsets mask the columns beyond n, fetched here.
+    auto epilogue = [&](int t, v4f acc, const Pre& pre) __attribute__((always_inline)) {
         const int n0 = t * 16 + 4 * lg;
-        if (mrow >= a.m || n0 >= a.n) return;
-        uint16_t* const drow = D + (long)mrow * a.n;
-        const bool vec = ((a.n & 3) == 0);  // then n0 + 3 < n and the 8-byte access is aligned
-        uint32_t old[4] = {0u, 0u, 0u, 0u};
-        float sb[4] = {1.f, 1.f, 1.f, 1.f};
+        const bool live = mrow < a.m && n0 < a.n;
+        const uint32_t d_off = ((uint32_t)mrow * (uint32_t)a.n + (uint32_t)n0) * 2u;
+        uint32_t old[4];
+        v4f sb;
+        uint32_t off[4];
+        if (vec) {
+            sb = __builtin_bit_cast(v4f, pre.sb);  // (a bit_cast of a single vector element would read element 0)
+            old[0] = (uint32_t)pre.d[0] & 0xffffu; old[1] = (uint32_t)pre.d[0] >> 16;
+            old[2] = (uint32_t)pre.d[1] & 0xffffu; old[3] = (uint32_t)pre.d[1] >> 16;
+        } else {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int n = min(n0 + v, a.n - 1);
-            if (a.scale_b && a.sb_stride) sb[v] = a.scale_b[n];
-        }
-        if (a.accumulate) {
-            if (vec) {
-                const uint2 q = *reinterpret_cast<const uint2*>(drow + n0);
-                old[0] = q.x & 0xffffu; old[1] = q.x >> 16; old[2] = q.y & 0xffffu; old[3] = q.y >> 16;
-            } else {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) old[v] = drow[min(n0 + v, a.n - 1)];
+            for (int v = 0; v < 4; ++v) {
+                off[v] = (live && n0 + v < a.n) ? d_off + 2u * v : kOutOfRange;
+                old[v] = a.accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(d_rsrc, (int)off[v], 0, 0) : 0u;
+                sb[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, (live && per_channel && n0 + v < a.n) ? (n0 + v) * 4 : (int)kOutOfRange, 0, 0));
             }
         }
         uint32_t o[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const float r = acc[v] * (sa * sb[v]);
+            const float r = acc[v] * (sa * (per_channel ? sb[v] : 1.0f));
             const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)old[v]) : load16<HFRK_F16>((uint16_t)old[v]);
             const float sum = a.accumulate ? base + r : r;
             o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
         }
         if (vec) {
-            *reinterpret_cast<uint2*>(drow + n0) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+            const v2i packed = {(int)(o[0] | (o[1] << 16)), (int)(o[2] | (o[3] << 16))};
+            __builtin_amdgcn_raw_buffer_store_b64(packed, d_rsrc, live ? (int)d_off : (int)kOutOfRange, 0, 0);
         } else {
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (n0 + v < a.n) drow[n0 + v] = (uint16_t)o[v];
+            for (int v = 0; v < 4; ++v) __builtin_amdgcn_raw_buffer_store_b16((short)o[v], d_rsrc, (int)off[v], 0, 0);
         }
     };
 
     // A wave's run is: [head segment] [whole row tiles ...] [last segment]; head/last may be partial tiles.
     const int tile_h = tile, kb_h = kc;
-    const int ke_h = (int)min((long)KC, (long)kb_h + count);
+    const int ke_h = min(KC, kb_h + count);
     const bool head_partial = count > 0 && !(kb_h == 0 && ke_h == KC);
-    const int tile_l = count > 0 ? (int)((w1 - 1) / KC) : -1;
-    const int ke_l = count > 0 ? (int)((w1 - 1) % KC) + 1 : 0;
+    const int tile_l = count > 0 ? (int)((w1 - 1) / (uint32_t)KC) : -1;
+    const int ke_l = count > 0 ? (int)((w1 - 1) - (uint32_t)tile_l * (uint32_t)KC) + 1 : 0;
     const bool last_distinct = count > 0 && tile_l != tile_h;
     const bool last_partial = last_distinct && ke_l != KC;
 
@@ -140,11 +160,15 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     v4f part_h = {0.f, 0.f, 0.f, 0.f};
 
     issue(count > 0);
+    // The scales are fetched behind the first chunk's requests: a wait for them up front would hold back the
+    // whole stream by one memory latency.
+    sa = a.scale_a[(long)min(mrow, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
     for (int i = 0; i < count; ++i) {
 #pragma unroll
         for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
 #pragma unroll
         for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + wr_off[t]) = wq[t];
+        pre_cur = pre_next;
         issue(i + 1 < count);  // registers are free again: request the next chunk before the LDS reads and MFMAs
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -163,7 +187,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
         __builtin_amdgcn_wave_barrier();
         if (++kc == KC) {  // a row tile ends inside this wave's run
             if (tile == tile_h && head_partial) part_h = acc;   // its first chunks belong to an earlier wave
-            else epilogue(tile, acc);                           // all of it was ours
+            else epilogue(tile, acc, pre_cur);                  // all of it was ours
             acc = v4f{0.f, 0.f, 0.f, 0.f};
             kc = 0;
             ++tile;
@@ -175,6 +199,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     if (single && head_partial && ke_h != KC) part_h = acc;
 
     // ---- combine the partial tiles of this workgroup ------------------------------------------------------------
+    // A segment that starts its tile inside this workgroup (first K chunk of the tile, or first chunk of the
+    // workgroup's range) makes this wave the one that finishes the tile.  Its D values are requested now, so that
+    // they arrive while the partial sums are exchanged.
+    const bool fin_h = head_partial && (kb_h == 0 || w0 == c0);
+    const Pre pre_h = prefetch(tile_h, fin_h);
+    const Pre pre_l = prefetch(tile_l, last_partial);
     // slot 0: head segment, slot 1: last segment (when it is another tile).  meta: tile (-1 = none), kb, ke.
     {
         int* const mine = meta + wv * 8;
@@ -182,52 +212,91 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
             mine[0] = head_partial ? tile_h : -1; mine[1] = kb_h; mine[2] = ke_h;
             mine[4] = last_partial ? tile_l : -1; mine[5] = 0;    mine[6] = ke_l;
         }
-        if (head_partial) slots[(wv * 2 + 0) * 64 + lane] = part_h;
-        if (last_partial) slots[(wv * 2 + 1) * 64 + lane] = acc;
+        if (head_partial) slots[wv * kSlotStride + lane] = part_h;
+        if (last_partial) slots[wv * kSlotStride + 64 + lane] = acc;
     }
     __syncthreads();
 
-    // A segment that starts its tile inside this workgroup (first K chunk of the tile, or first chunk of the
-    // workgroup's range) makes this wave the one that finishes the tile: add the following waves' head segments.
-    auto finish_segment = [&](int t, int kb, int ke, v4f sum) __attribute__((always_inline)) {
-        for (int j = wv + 1; j < kGemmWaves && ke < KC; ++j) {
-            const int* const mj = meta + j * 8;
-            if (mj[0] != t) {
-                if (mj[0] == -1 && mj[4] == -1 && mj[2] == mj[1]) continue;  // a wave without chunks
-                break;
+    // The finishing wave adds the following waves' head segments.  Every wave's description and head slot are
+    // fetched up front with independent LDS reads, and the two possible segments (head, last) share one copy of
+    // the code below: this part runs once per launch, with cold instruction fetch, so it is kept short.
+    if (!fin_h && !last_partial) return;
+    int m_tile = -1, m_kb = 0, m_ke = 0, m_last = -1;
+    if (lane < kGemmWaves) {
+        const v4i q = *reinterpret_cast<const v4i*>(meta + lane * 8);
+        m_tile = q[0]; m_kb = q[1]; m_ke = q[2];
+        m_last = meta[lane * 8 + 4];
+    }
+    v4f head_slot[kGemmWaves];
+#pragma unroll
+    for (int j = 1; j < kGemmWaves; ++j) head_slot[j] = slots[j * kSlotStride + lane];  // garbage where unused: never added
+    int w_tile[kGemmWaves], w_ke[kGemmWaves];
+    bool w_empty[kGemmWaves];
+#pragma unroll
+    for (int j = 1; j < kGemmWaves; ++j) {
+        w_tile[j] = __builtin_amdgcn_readlane(m_tile, j);
+        w_ke[j] = __builtin_amdgcn_readlane(m_ke, j);
+        w_empty[j] = w_tile[j] == -1 && __builtin_amdgcn_readlane(m_last, j) == -1 && w_ke[j] == __builtin_amdgcn_readlane(m_kb, j);
+    }
+    const int tile_c0 = (int)(c0 / (uint32_t)KC);
+#pragma unroll 1
+    for (int seg = 0; seg < 2; ++seg) {
+        if (!(seg == 0 ? fin_h : last_partial)) continue;
+        const int t = seg == 0 ? tile_h : tile_l;
+        const int kb = seg == 0 ? kb_h : 0;
+        int ke = seg == 0 ? ke_h : ke_l;
+        v4f sum = seg == 0 ? part_h : acc;
+        Pre pre;
+        pre.d = seg == 0 ? pre_h.d : pre_l.d;
+        pre.sb = seg == 0 ? pre_h.sb : pre_l.sb;
+        bool chain = true;
+#pragma unroll
+        for (int j = 1; j < kGemmWaves; ++j) {
+            if (j > wv && chain && ke < KC && !w_empty[j]) {  // a wave without chunks is skipped
+                if (w_tile[j] == t) {
+                    sum += head_slot[j];
+                    ke = w_ke[j];
+                } else {
+                    chain = false;
+                }
             }
-            sum += slots[(j * 2 + 0) * 64 + lane];
-            ke = mj[2];
         }
-        if (kb == 0 && ke == KC) {
-            epilogue(t, sum);
-            return;
+        if (!(kb == 0 && ke == KC)) {
+            // the tile continues in a neighbouring workgroup: park this workgroup's share, count the arrival
+            const int slot = (t == tile_c0) ? 0 : 1;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum), ws_rsrc, ((g * 2 + slot) * 64 + lane) * 16, 0, kCoherent);
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's store acknowledged before the arrival is counted
+            int last = 0;
+            if (lane == 0) {
+                const int mine = ke - kb;
+                const int seen = atomicAdd(&a.counters[t], mine);
+                last = (seen + mine == KC);
+                if (last) a.counters[t] = 0;  // ready for the next launch
+            }
+            last = __builtin_amdgcn_readfirstlane(last);
+            if (!last) continue;
+            // contributors are the workgroups whose chunk range meets [t*KC, (t+1)*KC), in id order; only the first
+            // of them can have the tile as its second (slot 1)
+            const uint32_t lo = (uint32_t)t * (uint32_t)KC, hi = lo + (uint32_t)KC;
+            const int g_first = (int)(((lo + 1) * (uint32_t)G + C - 1) / C) - 1;
+            const int g_last = (int)((hi * (uint32_t)G + C - 1) / C) - 1;
+            const int sl_first = ((uint32_t)g_first * C / (uint32_t)G == lo) ? 0 : 1;
+            sum = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+            for (int base = g_first; base <= g_last; base += 4) {
+                v4i q[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {  // four partials in flight; past the last one the load is out of range: zeros
+                    const int gg = base + u;
+                    const int sl = gg == g_first ? sl_first : 0;
+                    q[u] = __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, gg <= g_last ? ((gg * 2 + sl) * 64 + lane) * 16 : (int)kOutOfRange, 0, kCoherent);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) sum += __builtin_bit_cast(v4f, q[u]);
+            }
         }
-        // the tile continues in a neighbouring workgroup: park this workgroup's share, count the arrival
-        const int slot = (t == (int)(c0 / KC)) ? 0 : 1;
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum), ws_rsrc, ((g * 2 + slot) * 64 + lane) * 16, 0, kCoherent);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's store acknowledged before the arrival is counted
-        int last = 0;
-        if (lane == 0) {
-            const int mine = ke - kb;
-            const int seen = atomicAdd(&a.counters[t], mine);
-            last = (seen + mine == KC);
-            if (last) a.counters[t] = 0;  // ready for the next launch
-        }
-        last = __builtin_amdgcn_readfirstlane(last);
-        if (!last) return;
-        const long lo = (long)t * KC, hi = lo + KC;
-        const int g_first = (int)(((lo + 1) * G + C - 1) / C) - 1;
-        const int g_last = (int)((hi * G + C - 1) / C) - 1;
-        v4f total = {0.f, 0.f, 0.f, 0.f};
-        for (int gg = g_first; gg <= g_last; ++gg) {
-            const int sl = ((int)((gg * C / G) / KC) == t) ? 0 : 1;
-            total += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ((gg * 2 + sl) * 64 + lane) * 16, 0, kCoherent));
-        }
-        epilogue(t, total);
-    };
-    if (head_partial && (kb_h == 0 || w0 == c0)) finish_segment(tile_h, kb_h, ke_h, part_h);
-    if (last_partial) finish_segment(tile_l, 0, ke_l, acc);
+        epilogue(t, sum, pre);
+    }
 }
 
 int launch_stream_kernel(const GemmArgs& args, int act_loads, int lds_bytes, hipStream_t stream) {
