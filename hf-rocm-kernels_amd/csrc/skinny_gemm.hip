@@ -590,6 +590,8 @@ static int gemm_launch(const void* A, const void* B, void* D, const float* scale
     args.units = p.panels * p.slabs;
     args.grid = p.grid;
     args.nbuf = 2;
+    args.chunks_q = args.units / p.grid;
+    args.chunks_r = args.units % p.grid;
     args.ws = st->ws;
     args.counters = st->counters;
     // the vector store path needs 8-byte aligned rows

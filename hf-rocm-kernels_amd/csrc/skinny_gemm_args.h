@@ -23,12 +23,13 @@ struct GemmArgs {
     int m, n, k, b_stride;
     int d_dtype, accumulate;
     int panels, slabs, units, grid, nbuf;
+    int chunks_q, chunks_r;  // wave-stream kernel: (panels * slabs) / grid and % grid
     float* ws;
     int* counters;
 };
 
 // wave-stream kernel (m <= 16), skinny_gemm_stream.hip
 int launch_stream_kernel(const GemmArgs& args, int act_loads, int lds_bytes, hipStream_t stream);
-constexpr int kStreamLdsBytes = kGemmWaves * 2 * kTileBytes + 256;
+constexpr int kStreamLdsBytes = kGemmWaves * 2 * kTileBytes;
 
 }  // namespace hfrk

@@ -1,19 +1,26 @@
-// FP8 skinny GEMM, m <= 16: every wavefront streams its own run of weight chunks, nothing else is shared.
+// FP8 skinny GEMM, m <= 16: every wavefront streams its own run of weight chunks, nothing is shared in the loop.
 //
 // The weight matrix is cut into chunks of 16 rows x 256 K-bytes (4 KB), numbered row tile by row tile, K fastest.
-// The chunk sequence is split evenly over the workgroups and, inside a workgroup, evenly over its 8 waves, so a
-// wave owns one contiguous run: part of a row tile, then whole row tiles, then part of another.  For each chunk
-// the wave loads the 4 KB of weights (four 16-byte `nt` loads per lane, 4 rows x 256 contiguous bytes per
-// instruction) and the matching m x 256 bytes of activations (L1/L2 hits; rows >= m are out of range and cost
-// nothing), turns both into MFMA operand layout through two private, XOR-swizzled LDS tiles, and issues two
-// v_mfma_f32_16x16x128_f8f6f4.  The next chunk's loads are issued as soon as the registers have been copied to
-// LDS.  There is no barrier, no shared staging and no cross-wave dependency in the loop: measured, this loop
-// sustains the same bandwidth as a kernel that only reads the weights.
+// The chunk sequence is split evenly over the workgroups (the first `C % G` of them get one chunk more) and, inside
+// a workgroup, evenly over its 8 waves, so a wave owns one contiguous run: part of a row tile, then whole row
+// tiles, then part of another.  For each chunk the wave loads the 4 KB of weights (four 16-byte `nt` loads per
+// lane, 4 rows x 256 contiguous bytes per instruction) and the matching m x 256 bytes of activations (L1/L2 hits;
+// rows >= m are out of the buffer's range and cost no traffic), turns both into MFMA operand layout through two
+// private, XOR-swizzled LDS tiles, and issues two v_mfma_f32_16x16x128_f8f6f4.  The next chunk's loads are issued
+// as soon as the registers have been copied to LDS.  There is no barrier, no shared staging and no cross-wave
+// dependency in the loop: measured, this loop sustains the same bandwidth as a kernel that only reads the weights.
+//
+// What the decode shapes leave to optimise is serial instruction count: a launch lives 5-20 us, one wave retires
+// a few hundred instructions per microsecond, and both the code before the first load and the code after the last
+// MFMA sit on the critical path.  Hence the division-free chunk partition (quotient and remainder come from the
+// host), the early first request, and the closed-form reduction below that needs no exchanged descriptors.
 //
 // Sums that a wave cannot finish alone (a row tile split between waves) are combined once, after the loop:
-// partial 16x16 fp32 tiles go to LDS, one barrier, and the wave that holds a tile's first K chunk adds the others
-// in wave order.  A row tile split between workgroups goes through the workspace with a per-tile arrival counter;
-// the last workgroup to arrive adds the partials in workgroup order.  Both orders are fixed, so results are
+// a wave whose run starts inside a row tile leaves that partial 16x16 fp32 tile in LDS, one barrier, and the wave
+// that holds the tile's first chunk in this workgroup adds the partials of the waves after it whose runs start
+// before the tile (or the workgroup's range) ends -- wave runs are consecutive, so that is a comparison per wave.
+// A row tile split between workgroups goes through the workspace with a per-tile arrival counter; the last
+// workgroup to arrive adds the partials in workgroup order.  Both orders are fixed, so results are
 // bit-reproducible.  Scales, the optional accumulate-into-D and the single rounding to 16 bits happen there.
 //
 // Replaces, for m <= 16, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and
@@ -30,44 +37,62 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     constexpr int kCoherent = 17;  // sc0 | sc1
 
     extern __shared__ __align__(16) uint8_t lds[];
-    uint8_t* const tiles = lds;  // per wave: weight tile, activation tile
-    // After its loop a wave's tiles are dead; its two partial-sum slots (64 lanes x 16 bytes each) reuse the start of
-    // its own weight tile, so no other wave's data is touched before the barrier.
-    v4f* const slots = reinterpret_cast<v4f*>(lds);  // slot s of wave w at byte w*2*kTileBytes + s*1024
+    // After its loop a wave's tiles are dead; its partial-sum slot (64 lanes x 16 bytes) reuses the start of its own
+    // weight tile, so no other wave's data is touched before the barrier.
+    v4f* const slots = reinterpret_cast<v4f*>(lds);  // slot of wave w at byte w * 2 * kTileBytes
     constexpr int kSlotStride = 2 * kTileBytes / 16;  // in v4f
-    int* const meta = reinterpret_cast<int*>(lds + kGemmWaves * 2 * kTileBytes);  // [wave][2][tile,kb,ke,_]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
 
+    // ---- this wave's run of chunks (all 32-bit: the host checks (grid + 1) * chunks < 2^31) ------------------------
     const int G = a.grid;
-    const int KC = a.slabs;                      // 256-byte chunks per row tile
-    // All chunk arithmetic fits 32 bits: the host checks grid * chunks < 2^31 (64-bit division costs microseconds here).
-    const uint32_t C = (uint32_t)a.panels * (uint32_t)KC;  // all chunks
+    const int KC = a.slabs;  // 256-byte chunks per row tile
     const int b = blockIdx.x;
     const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;  // XCD x owns logical ids [x*G/8, (x+1)*G/8)
-    const uint32_t c0 = (uint32_t)g * C / (uint32_t)G, c1 = (uint32_t)(g + 1) * C / (uint32_t)G;
-    const uint32_t nwg = c1 - c0;
+    const uint32_t cq = (uint32_t)a.chunks_q, cr = (uint32_t)a.chunks_r;  // chunks / G, chunks % G
+    const uint32_t c0 = (uint32_t)g * cq + min((uint32_t)g, cr);
+    const uint32_t nwg = cq + ((uint32_t)g < cr ? 1u : 0u);
+    const uint32_t c1 = c0 + nwg;
     const uint32_t w0 = c0 + (uint32_t)wv * nwg / kGemmWaves, w1 = c0 + (uint32_t)(wv + 1) * nwg / kGemmWaves;
     const int count = (int)(w1 - w0);
+    int tile = (int)(w0 / (uint32_t)KC);  // chunk being multiplied
+    int kc = (int)(w0 - (uint32_t)tile * (uint32_t)KC);
 
+    // ---- first request, as early as possible ---------------------------------------------------------------------
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
+    const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
+    const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
+    v4i wq[4], aq[MA];
+    int itile = tile, ikc = kc;  // chunk being requested
+    auto issue_chunk = [&]() __attribute__((always_inline)) {
+        const uint32_t abase = (uint32_t)ikc * 256u;
+        const uint32_t wbase = (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)ikc * 256u;
+#pragma unroll
+        for (int t = 0; t < MA; ++t)
+            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+    };
+    if (count > 0) issue_chunk();
+    __builtin_amdgcn_sched_barrier(0);  // keep the set-up below behind the first request
+
+    // ---- the rest of the set-up -----------------------------------------------------------------------------------
     const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
     const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
     const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
     const bool vec = ((a.n & 3) == 0);  // then a lane's four outputs n0 .. n0+3 are all inside n and 8-byte aligned
     const bool per_channel = a.scale_b && a.sb_stride;
-
     const int mrow = li;  // the activation row (= output row) this lane's accumulator column belongs to
-    float sa = 1.0f;      // scale_a[row] * (scalar scale_b), loaded once the stream is under way
+    // The scales are fetched behind the first chunk's requests: a wait for them up front would hold back the whole
+    // stream by one memory latency.
+    const float sa = a.scale_a[(long)min(mrow, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
 
-    // ---- streaming loop ---------------------------------------------------------------------------------------
-    const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
-    const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
-    uint8_t* const tw = tiles + wv * 2 * kTileBytes;
+    uint8_t* const tw = lds + wv * 2 * kTileBytes;  // this wave's weight tile, then its activation tile
     uint8_t* const ta = tw + kTileBytes;
     int wr_off[4];
 #pragma unroll
@@ -80,32 +105,21 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     for (int h = 0; h < 2; ++h) rd_off[h] = li * 256 + ((((8 * h + 2 * lg) ^ li) & 15) << 4);
 
     // Old D values (accumulate mode) and per-channel scales of one row tile, requested ahead of the epilogue that
-    // uses them.  Only for the aligned case; out-of-range offsets make the loads free where they are not wanted.
+    // uses them (aligned n only).  Nothing is requested when nothing is wanted: even a load that is out of range
+    // and touches no memory returns in order, behind the CU's queue of real requests, and would be waited for.
     struct Pre { v2i d; v4i sb; };
+    const bool want_pre = vec && (a.accumulate || per_channel);
     auto prefetch = [&](int t, bool wanted) __attribute__((always_inline)) {
-        const int n0 = t * 16 + 4 * lg;
-        const bool ok = wanted && vec && li < a.m && n0 < a.n;
         Pre p;
-        p.d = __builtin_amdgcn_raw_buffer_load_b64(d_rsrc, (ok && a.accumulate) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
-        p.sb = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (ok && per_channel) ? n0 * 4 : (int)kOutOfRange, 0, 0);
+        p.d = v2i{0, 0};
+        p.sb = v4i{0, 0, 0, 0};
+        if (wanted && want_pre) {
+            const int n0 = t * 16 + 4 * lg;
+            const bool ok = li < a.m && n0 < a.n;
+            p.d = __builtin_amdgcn_raw_buffer_load_b64(d_rsrc, (ok && a.accumulate) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
+            p.sb = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (ok && per_channel) ? n0 * 4 : (int)kOutOfRange, 0, 0);
+        }
         return p;
-    };
-    Pre pre_next, pre_cur;
-    v4i wq[4], aq[MA];
-    int tile = (int)(w0 / (uint32_t)KC);             // chunk being multiplied
-    int kc = (int)(w0 - (uint32_t)tile * (uint32_t)KC);
-    int itile = tile, ikc = kc;                      // chunk being requested
-    auto issue = [&](bool in_range) __attribute__((always_inline)) {
-        const uint32_t abase = in_range ? (uint32_t)ikc * 256u : kOutOfRange;
-        const uint32_t wbase = in_range ? (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)ikc * 256u : kOutOfRange;
-#pragma unroll
-        for (int t = 0; t < MA; ++t)
-            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
-        pre_next = prefetch(itile, in_range && ikc == KC - 1);  // the chunk that ends a row tile brings the tile's D along
-        if (++ikc == KC) { ikc = 0; ++itile; }
     };
 
     // scale, add D (accumulate mode), round once, store: lane holds D^T[n0 + v][mrow], v = 0..3.
@@ -151,25 +165,22 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     const int tile_h = tile, kb_h = kc;
     const int ke_h = min(KC, kb_h + count);
     const bool head_partial = count > 0 && !(kb_h == 0 && ke_h == KC);
-    const int tile_l = count > 0 ? (int)((w1 - 1) / (uint32_t)KC) : -1;
-    const int ke_l = count > 0 ? (int)((w1 - 1) - (uint32_t)tile_l * (uint32_t)KC) + 1 : 0;
-    const bool last_distinct = count > 0 && tile_l != tile_h;
-    const bool last_partial = last_distinct && ke_l != KC;
 
+    // ---- streaming loop ---------------------------------------------------------------------------------------
+    Pre pre_next = prefetch(tile, count > 0 && kc == KC - 1), pre_cur;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     v4f part_h = {0.f, 0.f, 0.f, 0.f};
-
-    issue(count > 0);
-    // The scales are fetched behind the first chunk's requests: a wait for them up front would hold back the
-    // whole stream by one memory latency.
-    sa = a.scale_a[(long)min(mrow, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
     for (int i = 0; i < count; ++i) {
 #pragma unroll
         for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
 #pragma unroll
         for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + wr_off[t]) = wq[t];
         pre_cur = pre_next;
-        issue(i + 1 < count);  // registers are free again: request the next chunk before the LDS reads and MFMAs
+        if (i + 1 < count) {  // registers are free again: request the next chunk before the LDS reads and MFMAs
+            if (++ikc == KC) { ikc = 0; ++itile; }
+            issue_chunk();
+            pre_next = prefetch(itile, ikc == KC - 1);  // the chunk that ends a row tile brings the tile's D along
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -193,77 +204,48 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
             ++tile;
         }
     }
-    // here: acc = sums of the last segment if it is partial (else zero); part_h = head segment if it ended a tile.
-    // A run that lies inside one tile and does not end it leaves its only segment in acc: treat it as the head.
-    const bool single = count > 0 && !last_distinct;
-    if (single && head_partial && ke_h != KC) part_h = acc;
+    // Here (tile, kc) is the position behind the run.  kc != 0: the run ends inside row tile `tile`, whose first kc
+    // chunks are in acc -- unless the whole run lies inside that one tile, then they are the head segment.
+    const bool last_partial = count > 0 && kc != 0 && tile != tile_h;
+    const int tile_l = tile;
+    if (count > 0 && kc != 0 && tile == tile_h) part_h = acc;
 
     // ---- combine the partial tiles of this workgroup ------------------------------------------------------------
     // A segment that starts its tile inside this workgroup (first K chunk of the tile, or first chunk of the
     // workgroup's range) makes this wave the one that finishes the tile.  Its D values are requested now, so that
-    // they arrive while the partial sums are exchanged.
+    // they arrive while the partial sums are exchanged.  Every other head segment goes to the wave's slot; a wave
+    // without chunks leaves zeros there, so that the finishing wave can add by position alone.
     const bool fin_h = head_partial && (kb_h == 0 || w0 == c0);
     const Pre pre_h = prefetch(tile_h, fin_h);
     const Pre pre_l = prefetch(tile_l, last_partial);
-    // slot 0: head segment, slot 1: last segment (when it is another tile).  meta: tile (-1 = none), kb, ke.
-    {
-        int* const mine = meta + wv * 8;
-        if (lane == 0) {
-            mine[0] = head_partial ? tile_h : -1; mine[1] = kb_h; mine[2] = ke_h;
-            mine[4] = last_partial ? tile_l : -1; mine[5] = 0;    mine[6] = ke_l;
-        }
-        if (head_partial) slots[wv * kSlotStride + lane] = part_h;
-        if (last_partial) slots[wv * kSlotStride + 64 + lane] = acc;
-    }
+    if (!fin_h && (head_partial || count == 0)) slots[wv * kSlotStride + lane] = part_h;
     __syncthreads();
-
-    // The finishing wave adds the following waves' head segments.  Every wave's description and head slot are
-    // fetched up front with independent LDS reads, and the two possible segments (head, last) share one copy of
-    // the code below: this part runs once per launch, with cold instruction fetch, so it is kept short.
     if (!fin_h && !last_partial) return;
-    int m_tile = -1, m_kb = 0, m_ke = 0, m_last = -1;
-    if (lane < kGemmWaves) {
-        const v4i q = *reinterpret_cast<const v4i*>(meta + lane * 8);
-        m_tile = q[0]; m_kb = q[1]; m_ke = q[2];
-        m_last = meta[lane * 8 + 4];
-    }
+
+    // This part runs on one wave per row tile, after everything else: it is kept short, and the two possible
+    // segments (head, last) share one copy of the code.
     v4f head_slot[kGemmWaves];
 #pragma unroll
     for (int j = 1; j < kGemmWaves; ++j) head_slot[j] = slots[j * kSlotStride + lane];  // garbage where unused: never added
-    int w_tile[kGemmWaves], w_ke[kGemmWaves];
-    bool w_empty[kGemmWaves];
-#pragma unroll
-    for (int j = 1; j < kGemmWaves; ++j) {
-        w_tile[j] = __builtin_amdgcn_readlane(m_tile, j);
-        w_ke[j] = __builtin_amdgcn_readlane(m_ke, j);
-        w_empty[j] = w_tile[j] == -1 && __builtin_amdgcn_readlane(m_last, j) == -1 && w_ke[j] == __builtin_amdgcn_readlane(m_kb, j);
-    }
-    const int tile_c0 = (int)(c0 / (uint32_t)KC);
 #pragma unroll 1
     for (int seg = 0; seg < 2; ++seg) {
         if (!(seg == 0 ? fin_h : last_partial)) continue;
         const int t = seg == 0 ? tile_h : tile_l;
         const int kb = seg == 0 ? kb_h : 0;
-        int ke = seg == 0 ? ke_h : ke_l;
         v4f sum = seg == 0 ? part_h : acc;
         Pre pre;
         pre.d = seg == 0 ? pre_h.d : pre_l.d;
         pre.sb = seg == 0 ? pre_h.sb : pre_l.sb;
-        bool chain = true;
+        // the waves after this one whose runs start before the tile (or the workgroup's range) ends hold the rest
+        const uint32_t t_lo = (uint32_t)t * (uint32_t)KC;
+        const uint32_t t_end = min(t_lo + (uint32_t)KC, c1);
 #pragma unroll
-        for (int j = 1; j < kGemmWaves; ++j) {
-            if (j > wv && chain && ke < KC && !w_empty[j]) {  // a wave without chunks is skipped
-                if (w_tile[j] == t) {
-                    sum += head_slot[j];
-                    ke = w_ke[j];
-                } else {
-                    chain = false;
-                }
-            }
-        }
+        for (int j = 1; j < kGemmWaves; ++j)
+            if (j > wv && c0 + (uint32_t)j * nwg / kGemmWaves < t_end) sum += head_slot[j];
+        const int ke = (int)(t_end - t_lo);
         if (!(kb == 0 && ke == KC)) {
             // the tile continues in a neighbouring workgroup: park this workgroup's share, count the arrival
-            const int slot = (t == tile_c0) ? 0 : 1;
+            const int slot = (c0 >= t_lo) ? 0 : 1;  // slot 0: the tile holds this workgroup's first chunk
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum), ws_rsrc, ((g * 2 + slot) * 64 + lane) * 16, 0, kCoherent);
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's store acknowledged before the arrival is counted
             int last = 0;
@@ -275,12 +257,14 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
             }
             last = __builtin_amdgcn_readfirstlane(last);
             if (!last) continue;
-            // contributors are the workgroups whose chunk range meets [t*KC, (t+1)*KC), in id order; only the first
-            // of them can have the tile as its second (slot 1)
-            const uint32_t lo = (uint32_t)t * (uint32_t)KC, hi = lo + (uint32_t)KC;
-            const int g_first = (int)(((lo + 1) * (uint32_t)G + C - 1) / C) - 1;
-            const int g_last = (int)((hi * (uint32_t)G + C - 1) / C) - 1;
-            const int sl_first = ((uint32_t)g_first * C / (uint32_t)G == lo) ? 0 : 1;
+            // contributors are the workgroups whose chunk range meets [t_lo, t_lo + KC), in id order; only the first
+            // of them can have the tile as its second (slot 1).  owner(c) = the workgroup whose range holds chunk c.
+            auto owner = [&](uint32_t c) __attribute__((always_inline)) {
+                const uint32_t big = cr * (cq + 1u);  // chunks held by the first cr workgroups
+                return c < big ? (int)(c / (cq + 1u)) : (int)(cr + (c - big) / cq);
+            };
+            const int g_first = owner(t_lo), g_last = owner(t_lo + (uint32_t)KC - 1u);
+            const int sl_first = ((uint32_t)g_first * cq + min((uint32_t)g_first, cr) == t_lo) ? 0 : 1;
             sum = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 1
             for (int base = g_first; base <= g_last; base += 4) {

@@ -60,7 +60,7 @@ def all_plans(m, n, k):
     if m <= 16:  # wave-stream decomposition: grids that split row tiles between workgroups in different ways
         tiles, kc = (n + 15) // 16, k // 256
         for grid in sorted({min(256, tiles * kc), min(200, tiles * kc), min(7, tiles * kc), min(512, tiles * kc), 1}):
-            plans.append(_capi.GemmPlan(1, 0, 0, (m + 3) // 4, grid, tiles, kc, 8 * 2 * 4096 + 256))
+            plans.append(_capi.GemmPlan(1, 0, 0, (m + 3) // 4, grid, tiles, kc, 8 * 2 * 4096))
     for wn in (1, 2, 4, 8):
         wk = 8 // wn
         for ch in (1, 2):

@@ -63,14 +63,19 @@ SHAPES = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336), (10240, 8192
           (8192, 28672), (128, 256), (1000, 512), (50, 256), (13312, 16384), (2304, 16384)]
 
 
+def _stream_ranges(plan):
+    """Wave-stream decomposition: the first C % G workgroups hold C // G + 1 consecutive chunks, the others C // G."""
+    C, G = plan.panels * plan.slabs, plan.grid
+    q, r = divmod(C, G)
+    return [(g * q + min(g, r), g * q + min(g, r) + q + (1 if g < r else 0)) for g in range(G)]
+
+
 def _emulate_stream(plan):
-    """Wave-stream decomposition: chunks (row tile, K chunk) split over workgroups, then over their 8 waves."""
-    KC, T, G = plan.slabs, plan.panels, plan.grid
-    C = T * KC
-    cover = [0] * C
+    """Chunks (row tile, K chunk) split over workgroups, then over their 8 waves; who touches which row tile."""
+    KC, T = plan.slabs, plan.panels
+    cover = [0] * (T * KC)
     wg_of_tile = [[] for _ in range(T)]
-    for g in range(G):
-        c0, c1 = g * C // G, (g + 1) * C // G
+    for g, (c0, c1) in enumerate(_stream_ranges(plan)):
         assert c0 < c1
         n = c1 - c0
         for w in range(8):
@@ -79,6 +84,13 @@ def _emulate_stream(plan):
         for t in range(c0 // KC, (c1 - 1) // KC + 1):
             wg_of_tile[t].append(g)
     return cover, wg_of_tile
+
+
+def _stream_owner(plan, c):
+    """The kernel's closed form for the workgroup whose range holds chunk c."""
+    q, r = divmod(plan.panels * plan.slabs, plan.grid)
+    big = r * (q + 1)
+    return c // (q + 1) if c < big else r + (c - big) // q
 
 
 def _emulate(plan, n, k):
@@ -109,10 +121,10 @@ def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
         assert 1 <= plan.grid <= min(256, plan.panels * plan.slabs) and plan.lds_bytes <= 160 * 1024
         cover, wg_of_tile = _emulate_stream(plan)
         assert all(c == 1 for c in cover)
-        KC, G, C = plan.slabs, plan.grid, plan.panels * plan.slabs
+        KC = plan.slabs
         for t, who in enumerate(wg_of_tile):
             lo, hi = t * KC, (t + 1) * KC
-            assert who == list(range(((lo + 1) * G + C - 1) // C - 1, (hi * G + C - 1) // C)), (t, who)
+            assert who == list(range(_stream_owner(plan, lo), _stream_owner(plan, hi - 1) + 1)), (t, who)
         return
     assert m > 16
     assert plan.m_tiles == (m + 15) // 16 and plan.wn * plan.wk == 8 and plan.ch in (1, 2)
