@@ -444,6 +444,11 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     const long chunks = tiles * kc;
     long grid = chunks < kNumCU ? chunks : kNumCU;
     if (grid >= 8) grid -= grid % 8;  // whole XCD groups
+    // A grid that divides the row tiles keeps every tile inside one workgroup (no workspace round trip); worth it
+    // when it still fills at least three quarters of the CUs.
+    if (grid == kNumCU && tiles % kNumCU != 0)
+        for (long g = kNumCU - 8; g >= 3 * kNumCU / 4; g -= 8)
+            if (tiles % g == 0) { grid = g; break; }
     plan->m_tiles = 1;
     plan->wn = 0;
     plan->wk = 0;
