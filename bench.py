@@ -14,6 +14,10 @@ value       = algorithmic bytes of a step / time of a step, in GB/s (N*K + M*K +
 roofline    = the same bytes over the same HIP-event time, against 8 TB/s of HBM3E
 cpu_baseline= the oracle's torch path (dequantise -> fp32 matmul -> scale -> bf16) on the host cores, same shapes
 
+traffic     = HBM bytes per launch read back from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE runs of this
+              script with `--copy-calibration`, which appends a plain 256 MiB device copy whose counter reading
+              fixes the scale); the figure is a constant below because a benchmark cannot profile itself
+
 Prints one JSON line.  `--detail` adds a per-(shape, M) table measured outside the timed region.
 """
 import argparse
@@ -30,6 +34,10 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
 SHAPES = [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)]
 MS = [1, 2, 4, 8, 16]
 HBM_PEAK_GBPS = 8000.0
+# Mean HBM bytes per GEMM launch of a step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter runs
+# summarised in profiles/skinny_gemm_stream_llama3_8b_decode_hbm_traffic.txt: 1.0096 x the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 55223910
+CALIBRATION_COPY_BYTES = 256 << 20
 WORKLOAD = ("llama3-8b decode linears: M in {1,2,4,8,16} x qkv(6144,4096) o_proj(4096,4096) gate_up(28672,4096) "
             "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step")
 
@@ -177,6 +185,8 @@ def main():
     ap.add_argument("--detail", action="store_true", help="also time every (shape, M) case on its own")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed steps run a plain device copy of known size (for scaling rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -223,10 +233,19 @@ def main():
                    "weight_copies_per_shape": len(MS) * cycle, "timing": "HIP graph replay, HIP events",
                    "us_per_call_mean": round(ms_per_step * 1e3 / calls, 3), "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (all 20 launches of a step)",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "hfrk::skinny_gemm_stream_kernel<MA> (all 20 launches of a step)",
                      "bytes_per_launch": round(step_bytes / calls), "us_per_launch": round(ms_per_step * 1e3 / calls, 3)},
     }
+    if args.copy_calibration:
+        # bitwise_not over int32: one elementwise kernel that reads and writes CALIBRATION_COPY_BYTES each
+        src = torch.arange(CALIBRATION_COPY_BYTES // 4, dtype=torch.int32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.bitwise_not(src, out=dst)
+        torch.cuda.synchronize()
+        result["config"]["calibration_copy_bytes"] = CALIBRATION_COPY_BYTES
+        del src, dst
     if args.detail:
         result["cases"] = time_cases(torch, acts, weights, cycle)
     del graphs, weights, acts, outs
