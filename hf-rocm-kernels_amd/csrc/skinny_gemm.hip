@@ -417,93 +417,98 @@ constexpr int lds_bytes_for(int mt, int wk, int ch) {
     return kGemmWaves * kTileBytes + 2 * 16 * mt * (256 * wk * ch) + 16;
 }
 
-// Rough time model of one candidate decomposition, in nanoseconds; only its ordering matters.
-static double plan_cost(int n, int k, int mt, int wn, int wk, int ch, int* grid_out) {
-    const int bn = 16 * wn, ks = 256 * wk * ch;
-    const int panels = (n + bn - 1) / bn, slabs = k / ks;
-    const long units = (long)panels * slabs;
-    const int grid = (int)(units < kNumCU ? units : kNumCU);
-    *grid_out = grid;
-    const long upw = (units + grid - 1) / grid;                    // units of the busiest workgroup
-    const double cu_bw = 27.0;                                     // bytes/ns one CU sustains (~6.9 TB/s / 256)
-    const double stream = (double)upw * bn * ks / cu_bw;           // streaming time
-    const double per_unit = 120.0;                                 // barrier + slab staging exposure
-    const double panels_per_wg = (double)upw / slabs + 1.0;
-    const double flush = (wk > 1 ? 250.0 : 80.0) * panels_per_wg;  // in-workgroup reduction + store
-    const bool aligned = (units % grid == 0) && ((units / grid) % slabs == 0);
-    const double fixup = aligned ? 0.0 : 1500.0;                   // workspace round trip of shared panels
-    const double waste = (double)(panels * bn - n) / n;            // rows streamed past n cost no traffic but idle waves
-    return (stream + upw * per_unit + flush + fixup) * (1.0 + waste);
-}
-
-// m <= 16: every wave streams its own run of (16-row tile, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
-static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
-    const long tiles = (n + 15) / 16;
+// m <= 32: every wave streams its own run of (16*RT-row group, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
+static int fill_stream_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk_gemm_plan* plan) {
+    const int act_loads = (m + 3) / 4;
+    if (!stream_variant_exists(act_loads, row_tiles)) return HFRK_INVALID_CONFIG;
+    const long tiles = (n + 16 * row_tiles - 1) / (16 * row_tiles);
     if (tiles > kMaxPanels) return HFRK_BAD_SHAPE;
     const int kc = k / 256;
     const long chunks = tiles * kc;
-    long grid = chunks < kNumCU ? chunks : kNumCU;
+    long grid = grid_hint > 0 ? grid_hint : kNumCU;
+    if (grid > chunks) grid = chunks;
     if (grid >= 8) grid -= grid % 8;  // whole XCD groups
     // A grid that divides the row tiles keeps every tile inside one workgroup (no workspace round trip); worth it
     // when it still fills at least three quarters of the CUs.
-    if (grid == kNumCU && tiles % kNumCU != 0)
+    if (grid_hint <= 0 && grid == kNumCU && tiles % kNumCU != 0)
         for (long g = kNumCU - 8; g >= 3 * kNumCU / 4; g -= 8)
             if (tiles % g == 0) { grid = g; break; }
-    plan->m_tiles = 1;
+    plan->m_tiles = (act_loads + 3) / 4;
     plan->wn = 0;
-    plan->wk = 0;
-    plan->ch = (m + 3) / 4;
+    plan->wk = row_tiles;
+    plan->ch = act_loads;
     plan->grid = (int)grid;
     plan->panels = (int)tiles;
     plan->slabs = kc;
-    plan->lds_bytes = kStreamLdsBytes;
+    plan->lds_bytes = stream_lds_bytes(act_loads, row_tiles);
     return HFRK_SUCCESS;
 }
 
+static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    const int act_loads = (m + 3) / 4;
+    // Two row tiles per chunk halve the activation bytes pulled from L2 per weight byte: needed above 16 rows,
+    // worth it from 9 rows on once a wave's run still has a few 8 KB chunks.
+    int row_tiles = 1;
+    if (act_loads > 4) {
+        row_tiles = 2;
+    } else if (act_loads >= 3) {
+        const long chunks2 = (long)((n + 31) / 32) * (k / 256);
+        if (chunks2 >= (long)kStreamRt2MinChunksPerWave * kNumCU * kGemmWaves) row_tiles = 2;
+    }
+    return fill_stream_plan(m, n, k, row_tiles, 0, plan);
+}
+
+// Which decomposition for which shape.  The rules are measurements on MI355X over the Llama-3 8B/70B linears
+// (sweeps of every decomposition at m = 1..64), not a model:
+//   m <= 16          wave-stream kernel (activations per wave from L2: cheap up to 16 rows)
+//   m  > 16          workgroup kernel, which stages the activation slab once per workgroup in LDS:
+//                    4 row waves x 2 K waves almost everywhere; 2 x 4 for small weights (more K parallelism where a
+//                    workgroup only gets a few units); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (m <= 16) return make_stream_plan(m, n, k, plan);
     const int mt = (m + 15) / 16;
-    static const int wns[4] = {1, 2, 4, 8};
-    double best = 1e300;
-    bool found = false;
-    for (int wi = 0; wi < 4; ++wi) {
-        for (int ch = 2; ch >= 1; --ch) {
-            const int wn = wns[wi], wk = kGemmWaves / wn;
+    const double weight_mb = (double)n * k / 1.0e6;
+    int first = 4;
+    if (weight_mb < 48.0 && m <= 48) first = 2;
+    else if (weight_mb >= 200.0 && m > 48) first = 8;
+    const int prefs[3][4] = {{2, 4, 1, 8}, {4, 2, 8, 1}, {8, 4, 2, 1}};
+    const int* pref = first == 2 ? prefs[0] : first == 4 ? prefs[1] : prefs[2];
+    for (int pi = 0; pi < 4; ++pi) {
+        const int wn = pref[pi], wk = kGemmWaves / wn;
+        for (int ch = 1; ch <= 2; ++ch) {
             const int ks = 256 * wk * ch;
             if (k % ks != 0) continue;
             if (lds_bytes_for(mt, wk, ch) > kLdsLimit) continue;
             const int bn = 16 * wn;
             const long panels = (n + bn - 1) / bn;
             if (panels > kMaxPanels) continue;
-            int grid;
-            const double c = plan_cost(n, k, mt, wn, wk, ch, &grid);
-            if (c < best) {
-                best = c;
-                found = true;
-                plan->m_tiles = mt;
-                plan->wn = wn;
-                plan->wk = wk;
-                plan->ch = ch;
-                plan->grid = grid;
-                plan->panels = (int)panels;
-                plan->slabs = k / ks;
-                plan->lds_bytes = lds_bytes_for(mt, wk, ch);
-            }
+            const long units = panels * (k / ks);
+            plan->m_tiles = mt;
+            plan->wn = wn;
+            plan->wk = wk;
+            plan->ch = ch;
+            plan->grid = (int)(units < kNumCU ? units : kNumCU);
+            plan->panels = (int)panels;
+            plan->slabs = k / ks;
+            plan->lds_bytes = lds_bytes_for(mt, wk, ch);
+            return HFRK_SUCCESS;
         }
     }
-    return found ? HFRK_SUCCESS : HFRK_BAD_SHAPE;
+    return HFRK_BAD_SHAPE;
 }
 
 static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
-    if (p->wn == 0) {  // wave-stream decomposition
-        if (m > 16 || p->m_tiles != 1 || p->wk != 0 || p->ch < 1 || p->ch > 4 || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
-        if (p->panels != (n + 15) / 16 || p->slabs != k / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
+    if (p->wn == 0) {  // wave-stream decomposition: wk = row tiles per chunk, ch = activation loads
+        if (m > kStreamMaxM || !stream_variant_exists(p->ch, p->wk) || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
+        if (p->m_tiles != (p->ch + 3) / 4) return HFRK_INVALID_CONFIG;
+        const int rows = 16 * p->wk;
+        if (p->panels != (n + rows - 1) / rows || p->slabs != k / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
         const long chunks = (long)p->panels * p->slabs;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
         if (chunks * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's chunk arithmetic is 32-bit
-        if (p->lds_bytes != kStreamLdsBytes) return HFRK_INVALID_CONFIG;
+        if (p->lds_bytes != stream_lds_bytes(p->ch, p->wk)) return HFRK_INVALID_CONFIG;
         return HFRK_SUCCESS;
     }
     if (p->m_tiles < 1 || p->m_tiles > 4 || p->m_tiles * 16 < m) return HFRK_INVALID_CONFIG;
@@ -604,7 +609,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const float* scale
         // D rows would be misaligned for 8-byte stores: report rather than take a slow path silently
         return HFRK_BAD_ALIGNMENT;
     }
-    if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.lds_bytes, stream);
+    if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, p.lds_bytes, stream);
     switch (p.m_tiles) {
         case 1: return launch_mt<1>(args, p, stream);
         case 2: return launch_mt<2>(args, p, stream);

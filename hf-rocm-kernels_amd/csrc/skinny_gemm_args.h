@@ -23,13 +23,21 @@ struct GemmArgs {
     int m, n, k, b_stride;
     int d_dtype, accumulate;
     int panels, slabs, units, grid, nbuf;
-    int chunks_q, chunks_r;  // wave-stream kernel: (panels * slabs) / grid and % grid
+    int chunks_q, chunks_r;  // stream kernel: (panels * slabs) / grid and % grid
     float* ws;
     int* counters;
 };
 
-// wave-stream kernel (m <= 16), skinny_gemm_stream.hip
-int launch_stream_kernel(const GemmArgs& args, int act_loads, int lds_bytes, hipStream_t stream);
-constexpr int kStreamLdsBytes = kGemmWaves * 2 * kTileBytes;
+// wave-stream kernel (m <= 32), skinny_gemm_stream.hip: act_loads = ceil(m/4) 16-byte activation loads per lane and
+// chunk, row_tiles = 16-row weight tiles per chunk (1: act_loads 1..4; 2: act_loads 3..8)
+int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream);
+constexpr int kStreamMaxM = 32;
+constexpr int kStreamRt2MinChunksPerWave = 4;  // 9 <= m <= 16: two row tiles per chunk only if runs stay this long
+constexpr int stream_lds_bytes(int act_loads, int row_tiles) {
+    return kGemmWaves * (row_tiles + (act_loads + 3) / 4) * kTileBytes;
+}
+constexpr bool stream_variant_exists(int act_loads, int row_tiles) {
+    return (row_tiles == 1 && act_loads >= 1 && act_loads <= 4) || (row_tiles == 2 && act_loads >= 3 && act_loads <= 8);
+}
 
 }  // namespace hfrk

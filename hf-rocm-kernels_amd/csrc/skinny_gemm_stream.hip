@@ -1,12 +1,15 @@
-// FP8 skinny GEMM, m <= 16: every wavefront streams its own run of weight chunks, nothing is shared in the loop.
+// FP8 skinny GEMM, m <= 32: every wavefront streams its own run of weight chunks, nothing is shared in the loop.
 //
-// The weight matrix is cut into chunks of 16 rows x 256 K-bytes (4 KB), numbered row tile by row tile, K fastest.
+// The weight matrix is cut into chunks of 16*RT rows x 256 K-bytes (RT = 1 or 2 row tiles of 16 rows: 4 or 8 KB),
+// numbered row group by row group, K fastest.  ("Row tile" below means such a group of RT tiles.)
 // The chunk sequence is split evenly over the workgroups (the first `C % G` of them get one chunk more) and, inside
 // a workgroup, evenly over its 8 waves, so a wave owns one contiguous run: part of a row tile, then whole row
-// tiles, then part of another.  For each chunk the wave loads the 4 KB of weights (four 16-byte `nt` loads per
-// lane, 4 rows x 256 contiguous bytes per instruction) and the matching m x 256 bytes of activations (L1/L2 hits;
-// rows >= m are out of the buffer's range and cost no traffic), turns both into MFMA operand layout through two
-// private, XOR-swizzled LDS tiles, and issues two v_mfma_f32_16x16x128_f8f6f4.  The next chunk's loads are issued
+// tiles, then part of another.  For each chunk the wave loads the weights (4*RT 16-byte `nt` loads per lane, 4 rows
+// x 256 contiguous bytes per instruction) and the matching m x 256 bytes of activations (L1/L2 hits; rows >= m are
+// out of the buffer's range and cost no traffic), turns both into MFMA operand layout through private,
+// XOR-swizzled LDS tiles, and issues 2*RT*MT v_mfma_f32_16x16x128_f8f6f4 (MT = 16-row activation tiles).  RT = 2
+// halves the activation bytes read from L2 per weight byte, which is what limits m >= 16; for small m a 4 KB
+// chunk gives the short runs of the decode shapes more requests to overlap.  The next chunk's loads are issued
 // as soon as the registers have been copied to LDS.  There is no barrier, no shared staging and no cross-wave
 // dependency in the loop: measured, this loop sustains the same bandwidth as a kernel that only reads the weights.
 //
@@ -23,7 +26,7 @@
 // workgroup to arrive adds the partials in workgroup order.  Both orders are fixed, so results are
 // bit-reproducible.  Scales, the optional accumulate-into-D and the single rounding to 16 bits happen there.
 //
-// Replaces, for m <= 16, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and
+// Replaces, for m <= 32, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and
 // consumers (producers/n_full_tiles.cu:4-127, consumers/mfma_16x16x32_consumer.cu:1-168,
 // consumers/smfma_16x16x64_consumer.cu:1-158).
 #include "skinny_gemm_args.h"
@@ -31,16 +34,20 @@
 namespace hfrk {
 
 // MA = 16-byte activation loads per lane and chunk: load t brings rows 4t .. 4t+3, so 4*MA >= m.
-template <int MA>
+// RT = 16-row weight tiles per chunk.
+template <int MA, int RT>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const GemmArgs a) {
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kCoherent = 17;  // sc0 | sc1
+    constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles
+    constexpr int SUB = RT * MT;      // 16x16 output tiles per row group
+    constexpr int kWaveLds = (RT + MT) * kTileBytes;
 
     extern __shared__ __align__(16) uint8_t lds[];
-    // After its loop a wave's tiles are dead; its partial-sum slot (64 lanes x 16 bytes) reuses the start of its own
-    // weight tile, so no other wave's data is touched before the barrier.
-    v4f* const slots = reinterpret_cast<v4f*>(lds);  // slot of wave w at byte w * 2 * kTileBytes
-    constexpr int kSlotStride = 2 * kTileBytes / 16;  // in v4f
+    // After its loop a wave's tiles are dead; its partial-sum slots (SUB x 64 lanes x 16 bytes <= RT x 4 KB) reuse
+    // the start of its own weight tiles, so no other wave's data is touched before the barrier.
+    v4f* const slots = reinterpret_cast<v4f*>(lds);  // slot `sub` of wave w at v4f index w * kSlotStride + sub * 64
+    constexpr int kSlotStride = kWaveLds / 16;       // in v4f
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -66,16 +73,16 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
     const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
-    v4i wq[4], aq[MA];
+    v4i wq[4 * RT], aq[MA];
     int itile = tile, ikc = kc;  // chunk being requested
     auto issue_chunk = [&]() __attribute__((always_inline)) {
         const uint32_t abase = (uint32_t)ikc * 256u;
-        const uint32_t wbase = (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)ikc * 256u;
+        const uint32_t wbase = (uint32_t)itile * (16u * RT) * (uint32_t)a.b_stride + (uint32_t)ikc * 256u;
 #pragma unroll
         for (int t = 0; t < MA; ++t)
             aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < 4 * RT; ++t)
             wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
     };
     if (count > 0) issue_chunk();
@@ -87,13 +94,16 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
     const bool vec = ((a.n & 3) == 0);  // then a lane's four outputs n0 .. n0+3 are all inside n and 8-byte aligned
     const bool per_channel = a.scale_b && a.sb_stride;
-    const int mrow = li;  // the activation row (= output row) this lane's accumulator column belongs to
+    // Lane li holds the accumulator column of activation row (= output row) mt*16 + li of activation tile mt.
     // The scales are fetched behind the first chunk's requests: a wait for them up front would hold back the whole
     // stream by one memory latency.
-    const float sa = a.scale_a[(long)min(mrow, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+    float sa[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+        sa[mt] = a.scale_a[(long)min(mt * 16 + li, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
 
-    uint8_t* const tw = lds + wv * 2 * kTileBytes;  // this wave's weight tile, then its activation tile
-    uint8_t* const ta = tw + kTileBytes;
+    uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its MT activation tiles
+    uint8_t* const ta = tw + RT * kTileBytes;
     int wr_off[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -107,57 +117,76 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     // Old D values (accumulate mode) and per-channel scales of one row tile, requested ahead of the epilogue that
     // uses them (aligned n only).  Nothing is requested when nothing is wanted: even a load that is out of range
     // and touches no memory returns in order, behind the CU's queue of real requests, and would be waited for.
-    struct Pre { v2i d; v4i sb; };
+    struct Pre { v2i d[SUB]; v4i sb[RT]; };
     const bool want_pre = vec && (a.accumulate || per_channel);
     auto prefetch = [&](int t, bool wanted) __attribute__((always_inline)) {
         Pre p;
-        p.d = v2i{0, 0};
-        p.sb = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            p.sb[rt] = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) p.d[rt * MT + mt] = v2i{0, 0};
+        }
         if (wanted && want_pre) {
-            const int n0 = t * 16 + 4 * lg;
-            const bool ok = li < a.m && n0 < a.n;
-            p.d = __builtin_amdgcn_raw_buffer_load_b64(d_rsrc, (ok && a.accumulate) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
-            p.sb = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (ok && per_channel) ? n0 * 4 : (int)kOutOfRange, 0, 0);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const int n0 = (t * RT + rt) * 16 + 4 * lg;
+                p.sb[rt] = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (per_channel && n0 < a.n) ? n0 * 4 : (int)kOutOfRange, 0, 0);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const int mrow = mt * 16 + li;
+                    const bool ok = a.accumulate && mrow < a.m && n0 < a.n;
+                    p.d[rt * MT + mt] = __builtin_amdgcn_raw_buffer_load_b64(d_rsrc, ok ? (int)(((uint32_t)mrow * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
+                }
+            }
         }
         return p;
     };
 
-    // scale, add D (accumulate mode), round once, store: lane holds D^T[n0 + v][mrow], v = 0..3.
+    // scale, add D (accumulate mode), round once, store: lane holds D^T[n0 + v][mrow], v = 0..3, of every 16x16 tile.
     // Aligned n: D and the channel scales were prefetched (pre), one 8-byte store.  Ragged n (n % 4 != 0): 2-byte
     // buffer accesses whose out-of-range offsets mask the columns beyond n, fetched here.
-    auto epilogue = [&](int t, v4f acc, const Pre& pre) __attribute__((always_inline)) {
-        const int n0 = t * 16 + 4 * lg;
-        const bool live = mrow < a.m && n0 < a.n;
-        const uint32_t d_off = ((uint32_t)mrow * (uint32_t)a.n + (uint32_t)n0) * 2u;
-        uint32_t old[4];
-        v4f sb;
-        uint32_t off[4];
-        if (vec) {
-            sb = __builtin_bit_cast(v4f, pre.sb);  // (a bit_cast of a single vector element would read element 0)
-            old[0] = (uint32_t)pre.d[0] & 0xffffu; old[1] = (uint32_t)pre.d[0] >> 16;
-            old[2] = (uint32_t)pre.d[1] & 0xffffu; old[3] = (uint32_t)pre.d[1] >> 16;
-        } else {
+    auto epilogue = [&](int t, const v4f (&acc)[SUB], const Pre& pre) __attribute__((always_inline)) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                off[v] = (live && n0 + v < a.n) ? d_off + 2u * v : kOutOfRange;
-                old[v] = a.accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(d_rsrc, (int)off[v], 0, 0) : 0u;
-                sb[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, (live && per_channel && n0 + v < a.n) ? (n0 + v) * 4 : (int)kOutOfRange, 0, 0));
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int n0 = (t * RT + rt) * 16 + 4 * lg;
+                const int mrow = mt * 16 + li;
+                const bool live = mrow < a.m && n0 < a.n;
+                const uint32_t d_off = ((uint32_t)mrow * (uint32_t)a.n + (uint32_t)n0) * 2u;
+                uint32_t old[4];
+                v4f sb;
+                uint32_t off[4];
+                if (vec) {
+                    sb = __builtin_bit_cast(v4f, pre.sb[rt]);  // (a bit_cast of a single vector element would read element 0)
+                    const v2i d = pre.d[rt * MT + mt];
+                    old[0] = (uint32_t)d[0] & 0xffffu; old[1] = (uint32_t)d[0] >> 16;
+                    old[2] = (uint32_t)d[1] & 0xffffu; old[3] = (uint32_t)d[1] >> 16;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        off[v] = (live && n0 + v < a.n) ? d_off + 2u * v : kOutOfRange;
+                        old[v] = a.accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(d_rsrc, (int)off[v], 0, 0) : 0u;
+                        sb[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, (live && per_channel && n0 + v < a.n) ? (n0 + v) * 4 : (int)kOutOfRange, 0, 0));
+                    }
+                }
+                uint32_t o[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float r = acc[rt * MT + mt][v] * (sa[mt] * (per_channel ? sb[v] : 1.0f));
+                    const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)old[v]) : load16<HFRK_F16>((uint16_t)old[v]);
+                    const float sum = a.accumulate ? base + r : r;
+                    o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
+                }
+                if (vec) {
+                    const v2i packed = {(int)(o[0] | (o[1] << 16)), (int)(o[2] | (o[3] << 16))};
+                    __builtin_amdgcn_raw_buffer_store_b64(packed, d_rsrc, live ? (int)d_off : (int)kOutOfRange, 0, 0);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) __builtin_amdgcn_raw_buffer_store_b16((short)o[v], d_rsrc, (int)off[v], 0, 0);
+                }
             }
-        }
-        uint32_t o[4];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const float r = acc[v] * (sa * (per_channel ? sb[v] : 1.0f));
-            const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)old[v]) : load16<HFRK_F16>((uint16_t)old[v]);
-            const float sum = a.accumulate ? base + r : r;
-            o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
-        }
-        if (vec) {
-            const v2i packed = {(int)(o[0] | (o[1] << 16)), (int)(o[2] | (o[3] << 16))};
-            __builtin_amdgcn_raw_buffer_store_b64(packed, d_rsrc, live ? (int)d_off : (int)kOutOfRange, 0, 0);
-        } else {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) __builtin_amdgcn_raw_buffer_store_b16((short)o[v], d_rsrc, (int)off[v], 0, 0);
         }
     };
 
@@ -168,13 +197,14 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 
     // ---- streaming loop ---------------------------------------------------------------------------------------
     Pre pre_next = prefetch(tile, count > 0 && kc == KC - 1), pre_cur;
-    v4f acc = {0.f, 0.f, 0.f, 0.f};
-    v4f part_h = {0.f, 0.f, 0.f, 0.f};
+    v4f acc[SUB], part_h[SUB];
+#pragma unroll
+    for (int u = 0; u < SUB; ++u) acc[u] = part_h[u] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int i = 0; i < count; ++i) {
 #pragma unroll
-        for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
+        for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + (t / 4) * kTileBytes + wr_off[t % 4]) = aq[t];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + wr_off[t]) = wq[t];
+        for (int t = 0; t < 4 * RT; ++t) *reinterpret_cast<v4i*>(tw + (t / 4) * kTileBytes + wr_off[t % 4]) = wq[t];
         pre_cur = pre_next;
         if (i + 1 < count) {  // registers are free again: request the next chunk before the LDS reads and MFMAs
             if (++ikc == KC) { ikc = 0; ++itile; }
@@ -186,20 +216,36 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const v4i wlo = *reinterpret_cast<const v4i*>(tw + rd_off[h]);
-            const v4i whi = *reinterpret_cast<const v4i*>(tw + (rd_off[h] ^ 16));
-            const v4i alo = *reinterpret_cast<const v4i*>(ta + rd_off[h]);
-            const v4i ahi = *reinterpret_cast<const v4i*>(ta + (rd_off[h] ^ 16));
-            const v8i wop = {wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
-            const v8i aop = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
-            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc, 0, 0, 0, 0, 0, 0);
+            v8i wop[RT], aop[MT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const v4i lo = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + rd_off[h]);
+                const v4i hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
+                wop[rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const v4i lo = *reinterpret_cast<const v4i*>(ta + mt * kTileBytes + rd_off[h]);
+                const v4i hi = *reinterpret_cast<const v4i*>(ta + mt * kTileBytes + (rd_off[h] ^ 16));
+                aop[mt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[rt * MT + mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[rt], aop[mt], acc[rt * MT + mt], 0, 0, 0, 0, 0, 0);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (++kc == KC) {  // a row tile ends inside this wave's run
-            if (tile == tile_h && head_partial) part_h = acc;   // its first chunks belong to an earlier wave
-            else epilogue(tile, acc, pre_cur);                  // all of it was ours
-            acc = v4f{0.f, 0.f, 0.f, 0.f};
+            if (tile == tile_h && head_partial) {  // its first chunks belong to an earlier wave
+#pragma unroll
+                for (int u = 0; u < SUB; ++u) part_h[u] = acc[u];
+            } else {
+                epilogue(tile, acc, pre_cur);  // all of it was ours
+            }
+#pragma unroll
+            for (int u = 0; u < SUB; ++u) acc[u] = v4f{0.f, 0.f, 0.f, 0.f};
             kc = 0;
             ++tile;
         }
@@ -208,7 +254,10 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     // chunks are in acc -- unless the whole run lies inside that one tile, then they are the head segment.
     const bool last_partial = count > 0 && kc != 0 && tile != tile_h;
     const int tile_l = tile;
-    if (count > 0 && kc != 0 && tile == tile_h) part_h = acc;
+    if (count > 0 && kc != 0 && tile == tile_h) {
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) part_h[u] = acc[u];
+    }
 
     // ---- combine the partial tiles of this workgroup ------------------------------------------------------------
     // A segment that starts its tile inside this workgroup (first K chunk of the tile, or first chunk of the
@@ -218,35 +267,45 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     const bool fin_h = head_partial && (kb_h == 0 || w0 == c0);
     const Pre pre_h = prefetch(tile_h, fin_h);
     const Pre pre_l = prefetch(tile_l, last_partial);
-    if (!fin_h && (head_partial || count == 0)) slots[wv * kSlotStride + lane] = part_h;
+    if (!fin_h && (head_partial || count == 0)) {
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) slots[wv * kSlotStride + u * 64 + lane] = part_h[u];
+    }
     __syncthreads();
     if (!fin_h && !last_partial) return;
 
     // This part runs on one wave per row tile, after everything else: it is kept short, and the two possible
     // segments (head, last) share one copy of the code.
-    v4f head_slot[kGemmWaves];
-#pragma unroll
-    for (int j = 1; j < kGemmWaves; ++j) head_slot[j] = slots[j * kSlotStride + lane];  // garbage where unused: never added
 #pragma unroll 1
     for (int seg = 0; seg < 2; ++seg) {
         if (!(seg == 0 ? fin_h : last_partial)) continue;
         const int t = seg == 0 ? tile_h : tile_l;
         const int kb = seg == 0 ? kb_h : 0;
-        v4f sum = seg == 0 ? part_h : acc;
-        Pre pre;
-        pre.d = seg == 0 ? pre_h.d : pre_l.d;
-        pre.sb = seg == 0 ? pre_h.sb : pre_l.sb;
         // the waves after this one whose runs start before the tile (or the workgroup's range) ends hold the rest
         const uint32_t t_lo = (uint32_t)t * (uint32_t)KC;
         const uint32_t t_end = min(t_lo + (uint32_t)KC, c1);
+        v4f sum[SUB];
+        Pre pre;
 #pragma unroll
-        for (int j = 1; j < kGemmWaves; ++j)
-            if (j > wv && c0 + (uint32_t)j * nwg / kGemmWaves < t_end) sum += head_slot[j];
+        for (int rt = 0; rt < RT; ++rt) pre.sb[rt] = seg == 0 ? pre_h.sb[rt] : pre_l.sb[rt];
+#pragma unroll
+        for (int u = 0; u < SUB; ++u) {
+            pre.d[u] = seg == 0 ? pre_h.d[u] : pre_l.d[u];
+            sum[u] = seg == 0 ? part_h[u] : acc[u];
+            v4f other[kGemmWaves];
+#pragma unroll
+            for (int j = 1; j < kGemmWaves; ++j) other[j] = slots[j * kSlotStride + u * 64 + lane];  // garbage where unused: never added
+#pragma unroll
+            for (int j = 1; j < kGemmWaves; ++j)
+                if (j > wv && c0 + (uint32_t)j * nwg / kGemmWaves < t_end) sum[u] += other[j];
+        }
         const int ke = (int)(t_end - t_lo);
         if (!(kb == 0 && ke == KC)) {
             // the tile continues in a neighbouring workgroup: park this workgroup's share, count the arrival
             const int slot = (c0 >= t_lo) ? 0 : 1;  // slot 0: the tile holds this workgroup's first chunk
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum), ws_rsrc, ((g * 2 + slot) * 64 + lane) * 16, 0, kCoherent);
+#pragma unroll
+            for (int u = 0; u < SUB; ++u)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum[u]), ws_rsrc, (((g * 2 + slot) * SUB + u) * 64 + lane) * 16, 0, kCoherent);
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's store acknowledged before the arrival is counted
             int last = 0;
             if (lane == 0) {
@@ -265,49 +324,63 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
             };
             const int g_first = owner(t_lo), g_last = owner(t_lo + (uint32_t)KC - 1u);
             const int sl_first = ((uint32_t)g_first * cq + min((uint32_t)g_first, cr) == t_lo) ? 0 : 1;
-            sum = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < SUB; ++u) sum[u] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 1
             for (int base = g_first; base <= g_last; base += 4) {
-                v4i q[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {  // four partials in flight; past the last one the load is out of range: zeros
-                    const int gg = base + u;
-                    const int sl = gg == g_first ? sl_first : 0;
-                    q[u] = __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, gg <= g_last ? ((gg * 2 + sl) * 64 + lane) * 16 : (int)kOutOfRange, 0, kCoherent);
+                for (int u = 0; u < SUB; ++u) {
+                    v4i q[4];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {  // four partials in flight; past the last one the load is out of range: zeros
+                        const int gg = base + w;
+                        const int sl = gg == g_first ? sl_first : 0;
+                        q[w] = __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, gg <= g_last ? (((gg * 2 + sl) * SUB + u) * 64 + lane) * 16 : (int)kOutOfRange, 0, kCoherent);
+                    }
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) sum[u] += __builtin_bit_cast(v4f, q[w]);
                 }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) sum += __builtin_bit_cast(v4f, q[u]);
             }
         }
         epilogue(t, sum, pre);
     }
 }
 
-int launch_stream_kernel(const GemmArgs& args, int act_loads, int lds_bytes, hipStream_t stream) {
-#define HFRK_STREAM_CASE(MA_)                                                                                       \
-    case MA_: {                                                                                                     \
-        auto kern = skinny_gemm_stream_kernel<MA_>;                                                                 \
-        static bool attr_done[64] = {};                                                                             \
-        int dev = 0;                                                                                                \
-        HFRK_HIP_TRY(hipGetDevice(&dev));                                                                           \
-        if (dev >= 0 && dev < 64 && !attr_done[dev]) {                                                              \
-            HFRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                   \
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));               \
-            attr_done[dev] = true;                                                                                  \
-        }                                                                                                           \
-        hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);                     \
-        break;                                                                                                      \
+template <int MA, int RT>
+static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    auto kern = skinny_gemm_stream_kernel<MA, RT>;
+    static bool attr_done[64] = {};
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    if (dev >= 0 && dev < 64 && !attr_done[dev]) {
+        HFRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        attr_done[dev] = true;
     }
-    switch (act_loads) {
-        HFRK_STREAM_CASE(1)
-        HFRK_STREAM_CASE(2)
-        HFRK_STREAM_CASE(3)
-        HFRK_STREAM_CASE(4)
-        default: return HFRK_INVALID_CONFIG;
-    }
-#undef HFRK_STREAM_CASE
+    hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);
     HFRK_HIP_TRY(hipGetLastError());
     return HFRK_SUCCESS;
+}
+
+int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream) {
+    if (lds_bytes != stream_lds_bytes(act_loads, row_tiles)) return HFRK_INVALID_CONFIG;
+    if (row_tiles == 1) {
+        switch (act_loads) {
+            case 1: return launch_stream_one<1, 1>(args, lds_bytes, stream);
+            case 2: return launch_stream_one<2, 1>(args, lds_bytes, stream);
+            case 3: return launch_stream_one<3, 1>(args, lds_bytes, stream);
+            case 4: return launch_stream_one<4, 1>(args, lds_bytes, stream);
+        }
+    } else if (row_tiles == 2) {
+        switch (act_loads) {
+            case 3: return launch_stream_one<3, 2>(args, lds_bytes, stream);
+            case 4: return launch_stream_one<4, 2>(args, lds_bytes, stream);
+            case 5: return launch_stream_one<5, 2>(args, lds_bytes, stream);
+            case 6: return launch_stream_one<6, 2>(args, lds_bytes, stream);
+            case 7: return launch_stream_one<7, 2>(args, lds_bytes, stream);
+            case 8: return launch_stream_one<8, 2>(args, lds_bytes, stream);
+        }
+    }
+    return HFRK_INVALID_CONFIG;
 }
 
 }  // namespace hfrk

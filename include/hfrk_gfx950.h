@@ -47,15 +47,16 @@ enum hfrk_dtype { HFRK_F16 = 0, HFRK_BF16 = 1, HFRK_FP8_E4M3FN = 2 };
  * hfrk_skinny_gemm_ex() by an autotuner (counterpart of the knob table in
  * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102 and benchmarks/skinny_gemm/grid_search.py). */
 typedef struct hfrk_gemm_plan {
-    int m_tiles;   /* ceil(m/16): 16-row activation tiles kept in registers (1..4) */
-    int wn;        /* 0: wave-stream decomposition (m <= 16), every wave streams its own run of chunks.
+    int m_tiles;   /* ceil(m/16): 16-row activation tiles (wave-stream: 1..2, workgroup: 1..4) */
+    int wn;        /* 0: wave-stream decomposition (m <= 32), every wave streams its own run of chunks.
                       1,2,4,8: workgroup decomposition, wn waves spread over output rows (16 weight rows each) */
-    int wk;        /* workgroup decomposition: waves spread over K, wn*wk = 8.  wave-stream: 0 */
+    int wk;        /* workgroup decomposition: waves spread over K, wn*wk = 8.
+                      wave-stream: 16-row weight tiles per chunk, 1 (m <= 16) or 2 (9 <= m <= 32) */
     int ch;        /* workgroup decomposition: 256-byte K chunks each wave streams per slab (1 or 2).
                       wave-stream: 16-byte activation loads per lane and chunk, ceil(m/4) */
     int grid;      /* persistent workgroups launched */
-    int panels;    /* workgroup decomposition: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n/16) row tiles */
-    int slabs;     /* workgroup decomposition: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per tile */
+    int panels;    /* workgroup decomposition: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n / (16*wk)) row groups */
+    int slabs;     /* workgroup decomposition: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per group */
     int lds_bytes; /* dynamic LDS per workgroup */
 } hfrk_gemm_plan;
 

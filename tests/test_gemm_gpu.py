@@ -57,10 +57,14 @@ def all_plans(m, n, k):
     from hf_rocm_kernels import _capi
     mt = (m + 15) // 16
     plans = []
-    if m <= 16:  # wave-stream decomposition: grids that split row tiles between workgroups in different ways
-        tiles, kc = (n + 15) // 16, k // 256
-        for grid in sorted({min(256, tiles * kc), min(200, tiles * kc), min(7, tiles * kc), min(512, tiles * kc), 1}):
-            plans.append(_capi.GemmPlan(1, 0, 0, (m + 3) // 4, grid, tiles, kc, 8 * 2 * 4096))
+    if m <= 32:  # wave-stream decomposition: grids that split row groups between workgroups in different ways
+        ma, kc = (m + 3) // 4, k // 256
+        for rt in (1, 2):
+            if not ((rt == 1 and ma <= 4) or (rt == 2 and 3 <= ma <= 8)):
+                continue
+            groups = (n + 16 * rt - 1) // (16 * rt)
+            for grid in sorted({min(g, groups * kc) for g in (256, 200, 7, 512, 1)}):
+                plans.append(_capi.GemmPlan((ma + 3) // 4, 0, rt, ma, grid, groups, kc, 8 * (rt + (ma + 3) // 4) * 4096))
     for wn in (1, 2, 4, 8):
         wk = 8 // wn
         for ch in (1, 2):
@@ -90,7 +94,8 @@ def test_default_plan_matches_oracle(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
-                                   (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024)])
+                                   (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024),
+                                   (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096)])
 def test_every_plan_gives_the_same_answer(m, n, k):
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=7)

@@ -117,7 +117,9 @@ def _emulate(plan, n, k):
 def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
     plan = _capi.plan(m, n, k)
     if plan.wn == 0:  # m <= 16: wave-stream decomposition
-        assert m <= 16 and plan.ch == (m + 3) // 4 and plan.panels == -(-n // 16) and plan.slabs == k // 256
+        assert m <= 16 and plan.ch == (m + 3) // 4 and plan.m_tiles == (plan.ch + 3) // 4 and plan.slabs == k // 256
+        assert plan.wk in (1, 2) and (plan.wk == 2 or m <= 16) and plan.panels == -(-n // (16 * plan.wk))
+        assert plan.lds_bytes == 8 * (plan.wk + plan.m_tiles) * 4096
         assert 1 <= plan.grid <= min(256, plan.panels * plan.slabs) and plan.lds_bytes <= 160 * 1024
         cover, wg_of_tile = _emulate_stream(plan)
         assert all(c == 1 for c in cover)
