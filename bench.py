@@ -1,24 +1,33 @@
-"""Headline benchmark: FP8 skinny GEMM on Llama-3-8B decode linear shapes, one MI355X.
+"""Headline benchmark: FP8 skinny GEMM on Llama decode linear shapes, one MI355X.
 
-A step is one pass over BASELINE's second configuration: M in {1, 2, 4, 8, 16} x the four projection shapes
-qkv (6144, 4096), o_proj (4096, 4096), gate_up (28672, 4096), down (4096, 14336) -- 20 calls of
-`hf_rocm_kernels.skinny_gemm` (FP8 e4m3fn activations and weights, per-tensor scales, bf16 output accumulated
-into a zeroed buffer, as the reference's callers do).  All inputs are resident in HBM before the clock starts.
-Every call of a step reads a different copy of its weight, and a copy is read again only after ~1.5 GB of other
-weights have been streamed, so nothing is served from the 256 MB Infinity Cache or from L2.
+Default workload (`--workload llama3-8b`, BASELINE's second configuration): a step is one pass over
+M in {1, 2, 4, 8, 16} x the four projection shapes qkv (6144, 4096), o_proj (4096, 4096), gate_up (28672, 4096),
+down (4096, 14336) -- 20 calls of `hf_rocm_kernels.skinny_gemm` (FP8 e4m3fn activations and weights, per-tensor
+scales, bf16 output accumulated into a zeroed buffer, as the reference's callers do).  All inputs are resident in
+HBM before the clock starts.  Every call of a step reads a different copy of its weight, and a copy is read again
+only after more than a gigabyte of other weights has been streamed, so nothing is served from the 256 MB Infinity
+Cache or from L2.
+
+Other workloads, same method, for the remaining configurations:
+  llama3-70b  M in {1,4,8,16,32} x qkv (10240, 8192), o_proj (8192, 8192), gate_up (57344, 8192), down (8192, 28672)
+  scaled-m    M in {16,32,64} x (4096,4096), (28672,4096), (4096,14336) with per-token and per-channel scales
+              (`skinny_gemm_scaled`, activation rows 1 and M-1 drawn 20x larger)
+  mlp         the decoder MLP sub-block (`llama_mlp_combined_ops`: residual RMSNorm -> gate_up GEMM -> SwiGLU ->
+              down GEMM, output added to the residual), hidden 4096, M in {1, 8, 16}: 3 blocks = 12 launches per step
 
 The calls of a step are captured once into a HIP graph (the reference times its kernel the same way,
 operators/skinny_gemm/benchmarking_fn.py:62-92) so the figure is the GPU's, not the Python launch path's.
 
-value       = algorithmic bytes of a step / time of a step, in GB/s (N*K + M*K + 2*M*N + 4 bytes per call)
+value       = algorithmic bytes of a step / time of a step, in GB/s (GEMM: N*K + M*K + 2*M*N + 4*scales per call;
+              RMSNorm rows*cols*(2+2+2+1) + 2*cols; SwiGLU rows*n*(4+1))
 roofline    = the same bytes over the same HIP-event time, against 8 TB/s of HBM3E
 cpu_baseline= the oracle's torch path (dequantise -> fp32 matmul -> scale -> bf16) on the host cores, same shapes
-
 traffic     = HBM bytes per launch read back from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE runs of this
               script with `--copy-calibration`, which appends a plain 256 MiB device copy whose counter reading
               fixes the scale); the figure is a constant below because a benchmark cannot profile itself
 
-Prints one JSON line.  `--detail` adds a per-(shape, M) table measured outside the timed region.
+Prints one JSON line.  `--detail` adds a per-(shape, M) table measured outside the timed region, and for the GEMM
+workloads the cache-hot time of each case (one weight copy read over and over).
 """
 import argparse
 import json
@@ -31,61 +40,116 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-SHAPES = [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)]
-MS = [1, 2, 4, 8, 16]
 HBM_PEAK_GBPS = 8000.0
-# Mean HBM bytes per GEMM launch of a step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter runs
-# summarised in profiles/skinny_gemm_stream_llama3_8b_decode_hbm_traffic.txt: 1.0096 x the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 55223910
+# Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
+# runs summarised in profiles/skinny_gemm_stream_llama3_8b_decode_hbm_traffic.txt: 1.0096 x the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55223910}
 CALIBRATION_COPY_BYTES = 256 << 20
-WORKLOAD = ("llama3-8b decode linears: M in {1,2,4,8,16} x qkv(6144,4096) o_proj(4096,4096) gate_up(28672,4096) "
-            "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step")
+
+WORKLOADS = {
+    "llama3-8b": {
+        "shapes": [("qkv", 6144, 4096), ("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)],
+        "ms": [1, 2, 4, 8, 16], "cycle": 7, "scaled": False,
+        "text": "llama3-8b decode linears: M in {1,2,4,8,16} x qkv(6144,4096) o_proj(4096,4096) gate_up(28672,4096) "
+                "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
+        "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-8B decode shapes, M=1..16 (us/call in `cases`)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel<MA,RT> (all 20 launches of a step)",
+    },
+    "llama3-70b": {
+        "shapes": [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)],
+        "ms": [1, 4, 8, 16, 32], "cycle": 2, "scaled": False,
+        "text": "llama3-70b decode linears: M in {1,4,8,16,32} x qkv(10240,8192) o_proj(8192,8192) gate_up(57344,8192) "
+                "down(8192,28672); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
+        "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-70B decode shapes, M=1..32 (us/call in `cases`)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel<MA,RT> (M<=16), hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32)",
+    },
+    "scaled-m": {
+        "shapes": [("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)],
+        "ms": [16, 32, 64], "cycle": 8, "scaled": True,
+        "text": "M in {16,32,64} x (4096,4096) (28672,4096) (4096,14336); FP8 e4m3fn, per-token activation scales "
+                "(rows 1 and M-1 are 20x outliers) and per-output-channel weight scales, bf16 out; 9 calls per step",
+        "metric": "FP8 skinny-GEMM achieved HBM GB/s, per-token x per-channel scales, M=16..64 (us/call in `cases`)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel<4,RT> (M=16), hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64)",
+    },
+}
+MLP = {"hidden": 4096, "inter": 14336, "ms": [1, 8, 16], "cycle": 12, "eps": 1e-5,
+       "text": "llama3-8b decoder MLP sub-block (residual RMSNorm -> gate_up GEMM 28672x4096 -> SwiGLU -> down GEMM "
+               "4096x14336, + residual), M in {1,8,16}; 3 blocks = 12 launches per step",
+       "metric": "decoder MLP sub-block, achieved HBM GB/s over its four kernels (us/block in `cases`)"}
 
 
-def algorithmic_bytes(m, n, k):
-    return n * k + m * k + 2 * m * n + 4
+def gemm_bytes(m, n, k, n_scales=1):
+    return n * k + m * k + 2 * m * n + 4 * n_scales
 
 
-def make_inputs(torch, cycle):
-    """Activations per M, and 5*cycle quantised copies of each weight, all on the GPU."""
+def rms_bytes(rows, cols):
+    return rows * cols * (2 + 2 + 2 + 1) + 2 * cols
+
+
+def swiglu_bytes(rows, n):
+    return rows * n * (4 + 1)
+
+
+# ---- GEMM workloads ---------------------------------------------------------------------------------------------------
+
+def make_gemm_inputs(torch, spec):
+    """Activations per (M, K) and len(ms)*cycle quantised copies of each weight, all on the GPU."""
     from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
     gen = torch.Generator(device="cuda").manual_seed(0)
     acts, weights = {}, {}
-    for m in MS:
-        for _, n, k in SHAPES:
+    for m in spec["ms"]:
+        for _, n, k in spec["shapes"]:
             if (m, k) in acts:
                 continue
             a = torch.randn((m, k), generator=gen, device="cuda").to(torch.bfloat16).float()
-            sa = amax_scale(a)
-            acts[(m, k)] = (fp8_quantize(a, sa)[0], sa.reshape(1))
-    for name, n, k in SHAPES:
+            if spec["scaled"]:
+                a[1] *= 20.0
+                a[m - 1] *= 20.0
+                sa = amax_scale(a, dim=1)
+            else:
+                sa = amax_scale(a)
+            acts[(m, k)] = (fp8_quantize(a, sa)[0], sa.reshape(-1).contiguous())
+    for name, n, k in spec["shapes"]:
         copies = []
-        for _ in range(len(MS) * cycle):
+        for _ in range(len(spec["ms"]) * spec["cycle"]):
             w = torch.randn((n, k), generator=gen, device="cuda").mul_(0.02)
-            sw = amax_scale(w)
-            copies.append((fp8_quantize(w, sw)[0].t(), sw.reshape(1)))
+            sw = amax_scale(w, dim=1) if spec["scaled"] else amax_scale(w)
+            copies.append((fp8_quantize(w, sw)[0].t(), sw.reshape(-1).contiguous()))
             del w
         weights[name] = copies
     return acts, weights
 
 
-def capture_steps(torch, acts, weights, cycle):
-    """One HIP graph per step of the rotation; step i uses weight copy i*5 + (index of M)."""
+def gemm_caller(torch, spec, acts, weights):
+    """call(name, n, k, m, copy_index, out): one GEMM through the Python operator surface."""
     import hf_rocm_kernels
-    outs = {(m, n): torch.zeros((m, n), dtype=torch.bfloat16, device="cuda") for m in MS for _, n, _ in SHAPES}
+    if spec["scaled"]:
+        def call(name, n, k, m, ci, out):
+            w, sw = weights[name][ci]
+            a, sa = acts[(m, k)]
+            hf_rocm_kernels.skinny_gemm_scaled(a, w, sa, sw, output=out, accumulate=True)
+        return call
     scales = {}
-    for name, n, k in SHAPES:
-        for ci, (w, sw) in enumerate(weights[name]):
-            for m in MS:
+    for name, n, k in spec["shapes"]:
+        for ci, (_, sw) in enumerate(weights[name]):
+            for m in spec["ms"]:
                 scales[(name, ci, m)] = (acts[(m, k)][1] * sw).contiguous()
 
+    def call(name, n, k, m, ci, out):
+        # the op accumulates into `out`; zeroing belongs to the producer of the buffer
+        hf_rocm_kernels.skinny_gemm(acts[(m, k)][0], weights[name][ci][0], scales[(name, ci, m)], out)
+    return call
+
+
+def capture_gemm_steps(torch, spec, call):
+    """One HIP graph per step of the rotation; step i uses weight copy i*len(ms) + (index of M)."""
+    ms, shapes, cycle = spec["ms"], spec["shapes"], spec["cycle"]
+    outs = {(m, n): torch.zeros((m, n), dtype=torch.bfloat16, device="cuda") for m in ms for _, n, _ in shapes}
+
     def run_step(i):
-        for name, n, k in SHAPES:
-            for mi, m in enumerate(MS):
-                ci = i * len(MS) + mi
-                w, _ = weights[name][ci]
-                out = outs[(m, n)]  # the op accumulates into it; zeroing belongs to the producer of the buffer
-                hf_rocm_kernels.skinny_gemm(acts[(m, k)][0], w, scales[(name, ci, m)], out)
+        for name, n, k in shapes:
+            for mi, m in enumerate(ms):
+                call(name, n, k, m, i * len(ms) + mi, outs[(m, n)])
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -100,61 +164,70 @@ def capture_steps(torch, acts, weights, cycle):
     return graphs, outs
 
 
-def time_cases(torch, acts, weights, cycle, reps=40):
-    """Per-(shape, M) time from a graph of `5*cycle` calls over all copies of the weight, replayed `reps` times."""
-    import hf_rocm_kernels
+def time_graph(torch, g, calls, reps):
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        e1.synchronize()
+        ts.append(e0.elapsed_time(e1) * 1e3 / calls)
+    ts.sort()
+    return ts[len(ts) // 2], float(torch.tensor(ts).std())
+
+
+def time_gemm_cases(torch, spec, call, weights, reps=40):
+    """Per-(shape, M): time from a graph of one launch per weight copy (HBM-cold) and from a graph of 32 launches on
+    one copy (cache-hot: what the 256 MB Infinity Cache holds is not re-fetched from HBM)."""
     rows = []
     stream = torch.cuda.Stream()
-    for name, n, k in SHAPES:
-        for m in MS:
+    n_scales = lambda m, n: (m + n) if spec["scaled"] else 1
+    for name, n, k in spec["shapes"]:
+        copies = len(weights[name])
+        for m in spec["ms"]:
             out = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
-            a, sa = acts[(m, k)]
-            sc = [(sa * sw).contiguous() for _, sw in weights[name]]
             with torch.cuda.stream(stream):
-                hf_rocm_kernels.skinny_gemm(a, weights[name][0][0], sc[0], out)
+                call(name, n, k, m, 0, out)
             torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=stream):
-                for ci, (w, _) in enumerate(weights[name]):
-                    hf_rocm_kernels.skinny_gemm(a, w, sc[ci], out)
-            calls = len(weights[name])
-            for _ in range(3):
-                g.replay()
-            torch.cuda.synchronize()
-            ts = []
-            for _ in range(reps):
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                g.replay()
-                e1.record()
-                e1.synchronize()
-                ts.append(e0.elapsed_time(e1) * 1e3 / calls)
-            ts.sort()
-            us = ts[len(ts) // 2]
-            gbps = algorithmic_bytes(m, n, k) / us / 1e3
-            rows.append({"shape": name, "n": n, "k": k, "m": m, "us_per_call": round(us, 3),
-                         "us_std": round(float(torch.tensor(ts).std()), 3), "gbps": round(gbps, 1),
-                         "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4)})
-            del g
+            cold = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(cold, stream=stream):
+                for ci in range(copies):
+                    call(name, n, k, m, ci, out)
+            hot = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(hot, stream=stream):
+                for _ in range(32):
+                    call(name, n, k, m, 0, out)
+            us, std = time_graph(torch, cold, copies, reps)
+            us_hot, _ = time_graph(torch, hot, 32, reps)
+            gbps = gemm_bytes(m, n, k, n_scales(m, n)) / us / 1e3
+            rows.append({"shape": name, "n": n, "k": k, "m": m, "us_per_call": round(us, 3), "us_std": round(std, 3),
+                         "gbps": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                         "us_cache_hot": round(us_hot, 3)})
+            del cold, hot
     return rows
 
 
-def cpu_baseline(torch, budget_s=20.0):
-    """The oracle's reference path on the host: one pass over the same 20 (shape, M) cases, repeated while the
-    budget lasts (at least twice); median pass time.  Inputs are drawn on the CPU with the same recipe."""
+def cpu_baseline_gemm(torch, spec, budget_s):
+    """The oracle's reference path on the host: one pass over the same (shape, M) cases, repeated while the budget
+    lasts (at least twice); median pass time.  Inputs are drawn on the CPU with the same recipe."""
     from oracle import fp8 as ofp8
     from oracle import skinny_gemm as og
     torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1))))
     gen = torch.Generator().manual_seed(0)
     cases = []
-    for name, n, k in SHAPES:
+    for name, n, k in spec["shapes"]:
         w = torch.randn((n, k), generator=gen) * 0.02
-        sw = ofp8.amax_scale(w)
+        sw = ofp8.amax_scale(w, dim=1) if spec["scaled"] else ofp8.amax_scale(w)
         w8 = ofp8.fp8_quantize(w, sw)[0].t()
-        for m in MS:
+        for m in spec["ms"]:
             a = torch.randn((m, k), generator=gen).to(torch.bfloat16).float()
-            sa = ofp8.amax_scale(a)
-            cases.append((ofp8.fp8_quantize(a, sa)[0], w8, sa.reshape(1), sw.reshape(1), algorithmic_bytes(m, n, k)))
+            sa = ofp8.amax_scale(a, dim=1) if spec["scaled"] else ofp8.amax_scale(a)
+            cases.append((ofp8.fp8_quantize(a, sa)[0], w8, sa.reshape(-1), sw.reshape(-1),
+                          gemm_bytes(m, n, k, (m + n) if spec["scaled"] else 1)))
     total_bytes = sum(c[4] for c in cases)
 
     def one_pass():
@@ -172,17 +245,135 @@ def cpu_baseline(torch, budget_s=20.0):
     times.sort()
     med = times[len(times) // 2]
     return {"value": round(total_bytes / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "%d full passes over the same 20 (shape, M) cases, median pass %.3f s; oracle torch path "
-                      "dequantise->fp32 matmul->scale->bf16" % (len(times), med),
+            "sample": "%d full passes over the same %d (shape, M) cases, median pass %.3f s; oracle torch path "
+                      "dequantise->fp32 matmul->scale->bf16" % (len(times), len(cases), med),
             "ms_per_step": round(med * 1e3, 1)}
 
+
+# ---- MLP workload -----------------------------------------------------------------------------------------------------
+
+def mlp_block_bytes(m):
+    h, inter = MLP["hidden"], MLP["inter"]
+    return rms_bytes(m, h) + gemm_bytes(m, 2 * inter, h) + swiglu_bytes(m, inter) + gemm_bytes(m, h, inter)
+
+
+def make_mlp_inputs(torch):
+    from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    h, inter = MLP["hidden"], MLP["inter"]
+    copies = []
+    for _ in range(MLP["cycle"]):
+        wgu = torch.randn((2 * inter, h), generator=gen, device="cuda").mul_(0.02)
+        wd = torch.randn((h, inter), generator=gen, device="cuda").mul_(0.02)
+        sgu, sd = amax_scale(wgu), amax_scale(wd)
+        copies.append((fp8_quantize(wgu, sgu)[0].t(), sgu.reshape(1), fp8_quantize(wd, sd)[0].t(), sd.reshape(1)))
+        del wgu, wd
+    acts = {}
+    for m in MLP["ms"]:
+        x = torch.randn((m, h), generator=gen, device="cuda").to(torch.bfloat16)
+        res = torch.randn((m, h), generator=gen, device="cuda").to(torch.bfloat16)
+        acts[m] = (x, res)
+    rms_w = (1.0 + 0.1 * torch.randn((h,), generator=gen, device="cuda")).to(torch.bfloat16)
+    # static activation scales, as the reference's chain assumes: normalised activations ~ N(0,1), |swiglu| < 16
+    s_in = torch.full((1,), 6.0 / 448.0, device="cuda")
+    s_mid = torch.full((1,), 16.0 / 448.0, device="cuda")
+    return copies, acts, rms_w, s_in, s_mid
+
+
+def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid):
+    from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
+    out_scales = [((s_in * sgu).contiguous(), (s_mid * sd).contiguous()) for _, sgu, _, sd in copies]
+
+    def call(m, ci):
+        wgu, _, wd, _ = copies[ci]
+        x, res = acts[m]
+        return llama_mlp_combined_ops(x, res, rms_w, MLP["eps"], wgu, s_in, out_scales[ci][0], wd, s_mid,
+                                      out_scales[ci][1], add_residual=True)
+    return call
+
+
+def capture_mlp_steps(torch, call):
+    ms, cycle = MLP["ms"], MLP["cycle"]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for m in ms:
+            call(m, 0)
+    torch.cuda.synchronize()
+    graphs, keep = [], []
+    steps = cycle // len(ms)
+    for i in range(steps):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for mi, m in enumerate(ms):
+                keep.append(call(m, i * len(ms) + mi))
+        graphs.append(g)
+    return graphs, keep
+
+
+def time_mlp_cases(torch, call, reps=40):
+    rows = []
+    stream = torch.cuda.Stream()
+    for m in MLP["ms"]:
+        with torch.cuda.stream(stream):
+            call(m, 0)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        keep = []
+        with torch.cuda.graph(g, stream=stream):
+            for ci in range(MLP["cycle"]):
+                keep.append(call(m, ci))
+        us, std = time_graph(torch, g, MLP["cycle"], reps)
+        gbps = mlp_block_bytes(m) / us / 1e3
+        rows.append({"m": m, "us_per_block": round(us, 3), "us_std": round(std, 3), "gbps": round(gbps, 1),
+                     "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4)})
+        del g, keep
+    return rows
+
+
+def cpu_baseline_mlp(torch, budget_s):
+    from oracle import fp8 as ofp8
+    from oracle import llama_mlp as omlp
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1))))
+    gen = torch.Generator().manual_seed(0)
+    h, inter = MLP["hidden"], MLP["inter"]
+    wgu, wd = torch.randn((2 * inter, h), generator=gen) * 0.02, torch.randn((h, inter), generator=gen) * 0.02
+    sgu, sd = ofp8.amax_scale(wgu), ofp8.amax_scale(wd)
+    wgu8, wd8 = ofp8.fp8_quantize(wgu, sgu)[0].t(), ofp8.fp8_quantize(wd, sd)[0].t()
+    rms_w = (1.0 + 0.1 * torch.randn((h,), generator=gen)).to(torch.bfloat16)
+    s_in, s_mid = torch.full((1,), 6.0 / 448.0), torch.full((1,), 16.0 / 448.0)
+    cases = [(torch.randn((m, h), generator=gen).to(torch.bfloat16), torch.randn((m, h), generator=gen).to(torch.bfloat16))
+             for m in MLP["ms"]]
+    total_bytes = sum(mlp_block_bytes(m) for m in MLP["ms"])
+
+    def one_pass():
+        t0 = time.perf_counter()
+        for x, res in cases:
+            omlp.reference_llama_mlp(x, res.clone(), rms_w, MLP["eps"], wgu8, s_in, s_in * sgu, wd8, s_mid, s_mid * sd,
+                                     add_residual=True)
+        return time.perf_counter() - t0
+
+    one_pass()
+    times, spent = [], 0.0
+    while len(times) < 2 or (spent < budget_s and len(times) < 9):
+        t = one_pass()
+        times.append(t)
+        spent += t
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(total_bytes / med / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d full passes over the same 3 blocks, median pass %.3f s; oracle chain of the four torch "
+                      "reference functions" % (len(times), med), "ms_per_step": round(med * 1e3, 1)}
+
+
+# ---- main -------------------------------------------------------------------------------------------------------------
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--detail", action="store_true", help="also time every (shape, M) case on its own")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp"], default="llama3-8b")
+    ap.add_argument("--detail", action="store_true", help="also time every case on its own (HBM-cold and cache-hot)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -195,10 +386,24 @@ def main():
         sys.exit("bench.py needs a GPU (the kernels have no CPU path)")
     torch.cuda.set_device(0)
 
-    cycle = 7  # 35 copies of each weight: 7.6 GB in all, a copy is re-read after ~1.5 GB of other weights
-    acts, weights = make_inputs(torch, cycle)
-    graphs, outs = capture_steps(torch, acts, weights, cycle)
-    step_bytes = sum(algorithmic_bytes(m, n, k) for _, n, k in SHAPES for m in MS)
+    if args.workload == "mlp":
+        copies, acts, rms_w, s_in, s_mid = make_mlp_inputs(torch)
+        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid)
+        graphs, keep = capture_mlp_steps(torch, call)
+        step_bytes = sum(mlp_block_bytes(m) for m in MLP["ms"])
+        calls, text, metric = 4 * len(MLP["ms"]), MLP["text"], MLP["metric"]
+        kernel = "residual_rms_vec_kernel + skinny_gemm_stream_kernel + swiglu_vec_kernel + skinny_gemm_stream_kernel"
+        n_copies = MLP["cycle"]
+    else:
+        spec = WORKLOADS[args.workload]
+        acts, weights = make_gemm_inputs(torch, spec)
+        call = gemm_caller(torch, spec, acts, weights)
+        graphs, keep = capture_gemm_steps(torch, spec, call)
+        n_scales = (lambda m, n: m + n) if spec["scaled"] else (lambda m, n: 1)
+        step_bytes = sum(gemm_bytes(m, n, k, n_scales(m, n)) for _, n, k in spec["shapes"] for m in spec["ms"])
+        calls, text, metric, kernel = len(spec["shapes"]) * len(spec["ms"]), spec["text"], spec["metric"], spec["kernel"]
+        n_copies = len(spec["ms"]) * spec["cycle"]
+    cycle = len(graphs)
 
     for i in range(args.warmup):
         graphs[i % cycle].replay()
@@ -214,10 +419,9 @@ def main():
     gpu_ms = e0.elapsed_time(e1)
     ms_per_step = gpu_ms / args.steps
     gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
-    calls = len(SHAPES) * len(MS)
 
     result = {
-        "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-8B decode shapes, M=1..16 (us/call in `cases`)",
+        "metric": metric,
         "value": round(gbps, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -229,12 +433,12 @@ def main():
         "vs_baseline": None,
         "dtype": "fp8_e4m3fn",
         "data": "synthetic",
-        "config": {"workload": WORKLOAD, "calls_per_step": calls, "bytes_per_step": step_bytes,
-                   "weight_copies_per_shape": len(MS) * cycle, "timing": "HIP graph replay, HIP events",
+        "config": {"workload": text, "calls_per_step": calls, "bytes_per_step": step_bytes,
+                   "weight_copies_per_shape": n_copies, "timing": "HIP graph replay, HIP events",
                    "us_per_call_mean": round(ms_per_step * 1e3 / calls, 3), "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "hfrk::skinny_gemm_stream_kernel<MA> (all 20 launches of a step)",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                     "kernel": kernel,
                      "bytes_per_launch": round(step_bytes / calls), "us_per_launch": round(ms_per_step * 1e3 / calls, 3)},
     }
     if args.copy_calibration:
@@ -247,11 +451,19 @@ def main():
         result["config"]["calibration_copy_bytes"] = CALIBRATION_COPY_BYTES
         del src, dst
     if args.detail:
-        result["cases"] = time_cases(torch, acts, weights, cycle)
-    del graphs, weights, acts, outs
+        if args.workload == "mlp":
+            result["cases"] = time_mlp_cases(torch, call)
+        else:
+            result["cases"] = time_gemm_cases(torch, spec, call, weights)
+    del graphs, keep, call
+    if args.workload == "mlp":
+        del copies, acts
+    else:
+        del weights, acts
     torch.cuda.empty_cache()
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch, args.cpu_budget)
+        result["cpu_baseline"] = (cpu_baseline_mlp(torch, args.cpu_budget) if args.workload == "mlp"
+                                  else cpu_baseline_gemm(torch, spec, args.cpu_budget))
     print(json.dumps(result))
 
 
