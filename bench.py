@@ -14,6 +14,8 @@ Other workloads, same method, for the remaining configurations:
               (`skinny_gemm_scaled`, activation rows 1 and M-1 drawn 20x larger)
   mlp         the decoder MLP sub-block (`llama_mlp_combined_ops`: residual RMSNorm -> gate_up GEMM -> SwiGLU ->
               down GEMM, output added to the residual), hidden 4096, M in {1, 8, 16}: 3 blocks = 12 launches per step
+  mlp-fused   the same block in three launches: RMSNorm, gate_up GEMM with SwiGLU epilogue, down GEMM reading the
+              residual as its addend (`llama_mlp_combined_ops(..., fused=True)`)
 
 The calls of a step are captured once into a HIP graph (the reference times its kernel the same way,
 operators/skinny_gemm/benchmarking_fn.py:62-92) so the figure is the GPU's, not the Python launch path's.
@@ -280,7 +282,7 @@ def make_mlp_inputs(torch):
     return copies, acts, rms_w, s_in, s_mid
 
 
-def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid):
+def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused):
     from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
     out_scales = [((s_in * sgu).contiguous(), (s_mid * sd).contiguous()) for _, sgu, _, sd in copies]
 
@@ -288,7 +290,7 @@ def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid):
         wgu, _, wd, _ = copies[ci]
         x, res = acts[m]
         return llama_mlp_combined_ops(x, res, rms_w, MLP["eps"], wgu, s_in, out_scales[ci][0], wd, s_mid,
-                                      out_scales[ci][1], add_residual=True)
+                                      out_scales[ci][1], add_residual=True, fused=fused)
     return call
 
 
@@ -372,7 +374,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp"], default="llama3-8b")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused"], default="llama3-8b")
     ap.add_argument("--detail", action="store_true", help="also time every case on its own (HBM-cold and cache-hot)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
@@ -386,13 +388,18 @@ def main():
         sys.exit("bench.py needs a GPU (the kernels have no CPU path)")
     torch.cuda.set_device(0)
 
-    if args.workload == "mlp":
+    is_mlp = args.workload in ("mlp", "mlp-fused")
+    if is_mlp:
+        fused = args.workload == "mlp-fused"
         copies, acts, rms_w, s_in, s_mid = make_mlp_inputs(torch)
-        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid)
+        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused)
         graphs, keep = capture_mlp_steps(torch, call)
         step_bytes = sum(mlp_block_bytes(m) for m in MLP["ms"])
-        calls, text, metric = 4 * len(MLP["ms"]), MLP["text"], MLP["metric"]
-        kernel = "residual_rms_vec_kernel + skinny_gemm_stream_kernel + swiglu_vec_kernel + skinny_gemm_stream_kernel"
+        calls, text, metric = (3 if fused else 4) * len(MLP["ms"]), MLP["text"], MLP["metric"]
+        if fused:
+            text = text.replace("3 blocks = 12 launches", "fused into 3 launches per block: 3 blocks = 9 launches")
+        kernel = ("residual_rms_vec_kernel + skinny_gemm_stream_kernel<MA,2,swiglu> + skinny_gemm_stream_kernel" if fused else
+                  "residual_rms_vec_kernel + skinny_gemm_stream_kernel + swiglu_vec_kernel + skinny_gemm_stream_kernel")
         n_copies = MLP["cycle"]
     else:
         spec = WORKLOADS[args.workload]
@@ -451,18 +458,18 @@ def main():
         result["config"]["calibration_copy_bytes"] = CALIBRATION_COPY_BYTES
         del src, dst
     if args.detail:
-        if args.workload == "mlp":
+        if is_mlp:
             result["cases"] = time_mlp_cases(torch, call)
         else:
             result["cases"] = time_gemm_cases(torch, spec, call, weights)
     del graphs, keep, call
-    if args.workload == "mlp":
+    if is_mlp:
         del copies, acts
     else:
         del weights, acts
     torch.cuda.empty_cache()
     if not args.no_cpu:
-        result["cpu_baseline"] = (cpu_baseline_mlp(torch, args.cpu_budget) if args.workload == "mlp"
+        result["cpu_baseline"] = (cpu_baseline_mlp(torch, args.cpu_budget) if is_mlp
                                   else cpu_baseline_gemm(torch, spec, args.cpu_budget))
     print(json.dumps(result))
 

@@ -76,6 +76,12 @@ __device__ __forceinline__ uint8_t cvt_fp8(float a) {
     return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(a, a, 0u, false) & 0xffu);
 }
 
+// silu(g) * u * inv_scale in fp32, sigmoid as 1 / (1 + 2^(-g log2 e)) (the reference's form, swiglu_vectorized.cu:27-97)
+__device__ __forceinline__ float silu_mul(float g, float u, float inv_scale) {
+    const float e = __builtin_amdgcn_exp2f(-g * 1.44269504089f);
+    return g * __builtin_amdgcn_rcpf(1.0f + e) * u * inv_scale;
+}
+
 // Raw buffer resource over [base, base+bytes): loads beyond `bytes` return zero instead of faulting.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);

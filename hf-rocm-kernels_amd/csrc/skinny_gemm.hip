@@ -64,6 +64,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     uint16_t* const D = reinterpret_cast<uint16_t*>(a.D);
+    const uint16_t* const Dbase = reinterpret_cast<const uint16_t*>(a.base);  // added to the product when not null
+    const bool accumulate = a.base != nullptr;
 
     // ---- per-panel epilogue inputs, fetched when the panel's first weight loads are issued -------------------
     // The vector-memory counter retires in issue order, so a load issued at the end of a panel would wait for
@@ -89,8 +91,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         for (int mt = 0; mt < MT; ++mt) {
             dd[mt] = make_uint2(0u, 0u);
             const int mrow = mt * 16 + li;
-            if (a.accumulate && mrow < a.m) {
-                const uint16_t* const drow = D + (long)mrow * a.n;
+            if (accumulate && mrow < a.m) {
+                const uint16_t* const drow = Dbase + (long)mrow * a.n;
                 if (n_vec && n0 + 3 < a.n) {
                     dd[mt] = *reinterpret_cast<const uint2*>(drow + n0);
                 } else {
@@ -244,7 +246,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             for (int v = 0; v < 4; ++v) {
                 const float r = acc[mt][v] * (saq[mt] * (par ? sbq[1][v] : sbq[0][v]));
                 const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)oe[v]) : load16<HFRK_F16>((uint16_t)oe[v]);
-                const float sum = a.accumulate ? base + r : r;
+                const float sum = accumulate ? base + r : r;
                 o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
             }
             uint16_t* const drow = D + (long)mrow * a.n;
@@ -418,10 +420,10 @@ constexpr int lds_bytes_for(int mt, int wk, int ch) {
 }
 
 // m <= 32: every wave streams its own run of (16*RT-row group, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
-static int fill_stream_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk_gemm_plan* plan) {
+static int fill_stream_plan(int m, int n, int k, int row_tiles, bool swiglu, int grid_hint, hfrk_gemm_plan* plan) {
     const int act_loads = (m + 3) / 4;
-    if (!stream_variant_exists(act_loads, row_tiles)) return HFRK_INVALID_CONFIG;
-    const long tiles = (n + 16 * row_tiles - 1) / (16 * row_tiles);
+    if (!stream_variant_exists(act_loads, row_tiles, swiglu)) return HFRK_INVALID_CONFIG;
+    const long tiles = (n + 16 * row_tiles - 1) / (16 * row_tiles);  // swiglu: n/2 output columns in tiles of 16
     if (tiles > kMaxPanels) return HFRK_BAD_SHAPE;
     const int kc = k / 256;
     const long chunks = tiles * kc;
@@ -455,7 +457,7 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         const long chunks2 = (long)((n + 31) / 32) * (k / 256);
         if (chunks2 >= (long)kStreamRt2MinChunksPerWave * kNumCU * kGemmWaves) row_tiles = 2;
     }
-    return fill_stream_plan(m, n, k, row_tiles, 0, plan);
+    return fill_stream_plan(m, n, k, row_tiles, false, 0, plan);
 }
 
 // Which decomposition for which shape.  The rules are measurements on MI355X over the Llama-3 8B/70B linears
@@ -499,11 +501,12 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     return HFRK_BAD_SHAPE;
 }
 
-static int check_plan(int m, int n, int k, const hfrk_gemm_plan* p) {
+static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p) {
+    if (swiglu && p->wn != 0) return HFRK_INVALID_CONFIG;  // the fused epilogue exists in the wave-stream kernel only
     if (p->wn == 0) {  // wave-stream decomposition: wk = row tiles per chunk, ch = activation loads
-        if (m > kStreamMaxM || !stream_variant_exists(p->ch, p->wk) || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
+        if (m > kStreamMaxM || !stream_variant_exists(p->ch, p->wk, swiglu) || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
         if (p->m_tiles != (p->ch + 3) / 4) return HFRK_INVALID_CONFIG;
-        const int rows = 16 * p->wk;
+        const int rows = swiglu ? 16 : 16 * p->wk;  // with the SwiGLU epilogue n counts output columns: one gate + one up tile
         if (p->panels != (n + rows - 1) / rows || p->slabs != k / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
         const long chunks = (long)p->panels * p->slabs;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
@@ -552,27 +555,41 @@ static int launch_mt(const GemmArgs& args, const hfrk_gemm_plan& p, hipStream_t 
     return HFRK_INVALID_CONFIG;
 }
 
-static int gemm_launch(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
-                       const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
-                       int accumulate, const hfrk_gemm_plan* user_plan, hipStream_t stream) {
+// D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
+static int gemm_launch(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
+                       const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k, int b_stride,
+                       int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (d_dtype != HFRK_F16 && d_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
     if (!A || !B || !D || !scale_a) return HFRK_BAD_SHAPE;
     if ((sa_stride != 0 && sa_stride != 1) || (sb_stride != 0 && sb_stride != 1)) return HFRK_BAD_SHAPE;
+    if (epilogue != HFRK_EPILOGUE_NONE && epilogue != HFRK_EPILOGUE_SWIGLU) return HFRK_INVALID_CONFIG;
+    const bool swiglu = epilogue == HFRK_EPILOGUE_SWIGLU;
+    if (swiglu && (!out_scale || base || m > 16 || n % 32 != 0)) return HFRK_BAD_SHAPE;
     // every offset the kernel forms, including rows of the last (padded) panel, must stay below 2^31
     if (((long)n + 128) * b_stride + k >= (1L << 31) || (long)m * k >= (1L << 31)) return HFRK_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15 || (b_stride & 15)) return HFRK_BAD_ALIGNMENT;
-    if (reinterpret_cast<uintptr_t>(D) & 1) return HFRK_BAD_ALIGNMENT;
+    if (swiglu) {
+        if (reinterpret_cast<uintptr_t>(D) & 3) return HFRK_BAD_ALIGNMENT;  // 4 fp8 outputs per store
+    } else {
+        // the vector path needs 8-byte aligned rows: report rather than take a slow path silently
+        const uintptr_t both = reinterpret_cast<uintptr_t>(D) | reinterpret_cast<uintptr_t>(base);
+        if ((both & 1) || ((n & 3) == 0 && (both & 7))) return HFRK_BAD_ALIGNMENT;
+    }
 
     hfrk_gemm_plan p;
     if (user_plan) {
         p = *user_plan;
-        const int rc = check_plan(m, n, k, &p);
+        const int rc = check_plan(m, swiglu ? n / 2 : n, k, swiglu, &p);
         if (rc != HFRK_SUCCESS) return rc;
     } else {
-        const int rc = make_plan(m, n, k, &p);
+        const int rc = swiglu ? fill_stream_plan(m, n / 2, k, 1, false, 0, &p) : make_plan(m, n, k, &p);
         if (rc != HFRK_SUCCESS) return rc;
+        if (swiglu) {  // same chunk count as a one-tile plan over n/2 rows, but every chunk holds a gate and an up tile
+            p.wk = 2;
+            p.lds_bytes = stream_lds_bytes(p.ch, 2);
+        }
     }
 
     int dev = 0;
@@ -585,6 +602,8 @@ static int gemm_launch(const void* A, const void* B, void* D, const float* scale
     args.A = static_cast<const uint8_t*>(A);
     args.B = static_cast<const uint8_t*>(B);
     args.D = D;
+    args.base = base;
+    args.out_scale = out_scale;
     args.scale_a = scale_a;
     args.scale_b = scale_b;
     args.sa_stride = sa_stride;
@@ -594,7 +613,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const float* scale
     args.k = k;
     args.b_stride = b_stride;
     args.d_dtype = d_dtype;
-    args.accumulate = accumulate;
+    args.accumulate = base != nullptr;
     args.panels = p.panels;
     args.slabs = p.slabs;
     args.units = p.panels * p.slabs;
@@ -604,12 +623,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const float* scale
     args.chunks_r = args.units % p.grid;
     args.ws = st->ws;
     args.counters = st->counters;
-    // the vector store path needs 8-byte aligned rows
-    if ((reinterpret_cast<uintptr_t>(D) & 7) != 0 && (n & 3) == 0) {
-        // D rows would be misaligned for 8-byte stores: report rather than take a slow path silently
-        return HFRK_BAD_ALIGNMENT;
-    }
-    if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, p.lds_bytes, stream);
+    if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     switch (p.m_tiles) {
         case 1: return launch_mt<1>(args, p, stream);
         case 2: return launch_mt<2>(args, p, stream);
@@ -660,15 +674,22 @@ int hfrk_skinny_gemm(const void* A, const void* B, void* D, const float* scale_t
     const int rc = hfrk_skinny_gemm_validate(m, n, k, b_stride, split_k, A_producers, B_producers, consumers, a_lanes,
                                              b_lanes, qsize, op_m, ops);
     if (rc != HFRK_SUCCESS) return rc;
-    return hfrk::gemm_launch(A, B, D, scale_tensor, 0, nullptr, 0, m, n, k, b_stride, d_dtype, 1, nullptr,
-                             static_cast<hipStream_t>(stream));
+    return hfrk::gemm_launch(A, B, D, D, scale_tensor, 0, nullptr, 0, nullptr, m, n, k, b_stride, d_dtype,
+                             HFRK_EPILOGUE_NONE, nullptr, static_cast<hipStream_t>(stream));
 }
 
 int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
                         const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
                         int accumulate, const hfrk_gemm_plan* plan, void* stream) {
-    return hfrk::gemm_launch(A, B, D, scale_a, sa_stride, scale_b, sb_stride, m, n, k, b_stride, d_dtype, accumulate,
-                             plan, static_cast<hipStream_t>(stream));
+    return hfrk::gemm_launch(A, B, D, accumulate ? D : nullptr, scale_a, sa_stride, scale_b, sb_stride, nullptr, m, n, k,
+                             b_stride, d_dtype, HFRK_EPILOGUE_NONE, plan, static_cast<hipStream_t>(stream));
+}
+
+int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
+                           const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k,
+                           int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
+    return hfrk::gemm_launch(A, B, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, m, n, k, b_stride, d_dtype,
+                             epilogue, plan, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -17,6 +17,8 @@ struct GemmArgs {
     const uint8_t* A;
     const uint8_t* B;
     void* D;
+    const void* base;        // accumulate mode: the 16-bit [m,n] tensor added to the product (may be D itself); else null
+    const float* out_scale;  // SwiGLU epilogue: the fp8 output is divided by out_scale[0]
     const float* scale_a;
     const float* scale_b;
     int sa_stride, sb_stride;
@@ -30,14 +32,17 @@ struct GemmArgs {
 
 // wave-stream kernel (m <= 32), skinny_gemm_stream.hip: act_loads = ceil(m/4) 16-byte activation loads per lane and
 // chunk, row_tiles = 16-row weight tiles per chunk (1: act_loads 1..4; 2: act_loads 3..8)
-int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream);
+// swiglu: the weight holds gate rows [0, n/2) and up rows [n/2, n); a chunk pairs gate tile t with up tile t
+// (row_tiles must be 2) and the epilogue writes fp8(silu(gate) * up / out_scale) to D [m, n/2].
+int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream);
 constexpr int kStreamMaxM = 32;
 constexpr int kStreamRt2MinChunksPerWave = 4;  // 9 <= m <= 16: two row tiles per chunk only if runs stay this long
 constexpr int stream_lds_bytes(int act_loads, int row_tiles) {
     return kGemmWaves * (row_tiles + (act_loads + 3) / 4) * kTileBytes;
 }
-constexpr bool stream_variant_exists(int act_loads, int row_tiles) {
-    return (row_tiles == 1 && act_loads >= 1 && act_loads <= 4) || (row_tiles == 2 && act_loads >= 3 && act_loads <= 8);
+constexpr bool stream_variant_exists(int act_loads, int row_tiles, bool swiglu = false) {
+    return swiglu ? (row_tiles == 2 && act_loads >= 1 && act_loads <= 4)
+                  : (row_tiles == 1 && act_loads >= 1 && act_loads <= 4) || (row_tiles == 2 && act_loads >= 3 && act_loads <= 8);
 }
 
 }  // namespace hfrk

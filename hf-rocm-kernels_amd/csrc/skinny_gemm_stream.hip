@@ -35,13 +35,17 @@ namespace hfrk {
 
 // MA = 16-byte activation loads per lane and chunk: load t brings rows 4t .. 4t+3, so 4*MA >= m.
 // RT = 16-row weight tiles per chunk.
-template <int MA, int RT>
+// SWIGLU: the weight is a gate_up projection (gate rows [0, n/2), up rows [n/2, n)); a chunk pairs gate tile t with
+// up tile t (RT = 2) and the epilogue stores fp8(silu(gate) * up / out_scale) into D [m, n/2] instead of the two
+// 16-bit projections -- the SwiGLU kernel of csrc/op_src/swiglu/swiglu_vectorized.cu:27-97 as a GEMM epilogue.
+template <int MA, int RT, bool SWIGLU>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const GemmArgs a) {
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kCoherent = 17;  // sc0 | sc1
     constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles
     constexpr int SUB = RT * MT;      // 16x16 output tiles per row group
     constexpr int kWaveLds = (RT + MT) * kTileBytes;
+    static_assert(!SWIGLU || RT == 2, "the SwiGLU epilogue pairs one gate tile with one up tile");
 
     extern __shared__ __align__(16) uint8_t lds[];
     // After its loop a wave's tiles are dead; its partial-sum slots (SUB x 64 lanes x 16 bytes <= RT x 4 KB) reuse
@@ -77,22 +81,26 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     int itile = tile, ikc = kc;  // chunk being requested
     auto issue_chunk = [&]() __attribute__((always_inline)) {
         const uint32_t abase = (uint32_t)ikc * 256u;
-        const uint32_t wbase = (uint32_t)itile * (16u * RT) * (uint32_t)a.b_stride + (uint32_t)ikc * 256u;
+        // row group t: weight rows [16*RT*t, 16*RT*(t+1)), or with SWIGLU rows [16t, 16t+16) and n/2 + the same
+        const uint32_t wbase = (uint32_t)itile * (SWIGLU ? 16u : 16u * RT) * (uint32_t)a.b_stride + (uint32_t)ikc * 256u;
 #pragma unroll
         for (int t = 0; t < MA; ++t)
             aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
 #pragma unroll
         for (int t = 0; t < 4 * RT; ++t)
-            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(SWIGLU ? (t / 4) * (a.n >> 1) + 4 * (t % 4) : 4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
     };
     if (count > 0) issue_chunk();
     __builtin_amdgcn_sched_barrier(0);  // keep the set-up below behind the first request
 
     // ---- the rest of the set-up -----------------------------------------------------------------------------------
     const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
-    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
+    const int n_out = SWIGLU ? (a.n >> 1) : a.n;  // columns of D
+    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)n_out * (SWIGLU ? 1u : 2u));
+    const __amdgpu_buffer_rsrc_t base_rsrc = make_rsrc(a.base, a.base ? (uint32_t)a.m * (uint32_t)a.n * 2u : 0u);
+    const bool accumulate = !SWIGLU && a.base != nullptr;
     const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
-    const bool vec = ((a.n & 3) == 0);  // then a lane's four outputs n0 .. n0+3 are all inside n and 8-byte aligned
+    const bool vec = SWIGLU || ((a.n & 3) == 0);  // then a lane's four outputs n0 .. n0+3 are all inside n and aligned
     const bool per_channel = a.scale_b && a.sb_stride;
     // Lane li holds the accumulator column of activation row (= output row) mt*16 + li of activation tile mt.
     // The scales are fetched behind the first chunk's requests: a wait for them up front would hold back the whole
@@ -101,6 +109,11 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
         sa[mt] = a.scale_a[(long)min(mt * 16 + li, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+    float inv_out_scale = 1.0f;
+    if (SWIGLU) {
+        const float os = a.out_scale[0];
+        inv_out_scale = os != 0.f ? 1.0f / os : 1.0f;
+    }
 
     uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its MT activation tiles
     uint8_t* const ta = tw + RT * kTileBytes;
@@ -118,7 +131,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     // uses them (aligned n only).  Nothing is requested when nothing is wanted: even a load that is out of range
     // and touches no memory returns in order, behind the CU's queue of real requests, and would be waited for.
     struct Pre { v2i d[SUB]; v4i sb[RT]; };
-    const bool want_pre = vec && (a.accumulate || per_channel);
+    const bool want_pre = vec && (accumulate || per_channel);
     auto prefetch = [&](int t, bool wanted) __attribute__((always_inline)) {
         Pre p;
 #pragma unroll
@@ -130,13 +143,13 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
         if (wanted && want_pre) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                const int n0 = (t * RT + rt) * 16 + 4 * lg;
+                const int n0 = SWIGLU ? rt * (a.n >> 1) + t * 16 + 4 * lg : (t * RT + rt) * 16 + 4 * lg;  // weight row
                 p.sb[rt] = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (per_channel && n0 < a.n) ? n0 * 4 : (int)kOutOfRange, 0, 0);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     const int mrow = mt * 16 + li;
-                    const bool ok = a.accumulate && mrow < a.m && n0 < a.n;
-                    p.d[rt * MT + mt] = __builtin_amdgcn_raw_buffer_load_b64(d_rsrc, ok ? (int)(((uint32_t)mrow * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
+                    const bool ok = accumulate && mrow < a.m && n0 < a.n;
+                    p.d[rt * MT + mt] = __builtin_amdgcn_raw_buffer_load_b64(base_rsrc, ok ? (int)(((uint32_t)mrow * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
                 }
             }
         }
@@ -147,6 +160,30 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     // Aligned n: D and the channel scales were prefetched (pre), one 8-byte store.  Ragged n (n % 4 != 0): 2-byte
     // buffer accesses whose out-of-range offsets mask the columns beyond n, fetched here.
     auto epilogue = [&](int t, const v4f (&acc)[SUB], const Pre& pre) __attribute__((always_inline)) {
+        if constexpr (SWIGLU) {
+            // acc[0*MT+mt] = gate tile, acc[1*MT+mt] = up tile of the same output columns n0 .. n0+3
+            const int n0 = t * 16 + 4 * lg;
+            const v4f sbg = __builtin_bit_cast(v4f, pre.sb[0]), sbu = __builtin_bit_cast(v4f, pre.sb[1]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int mrow = mt * 16 + li;
+                float y[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    float g = acc[mt][v] * (sa[mt] * (per_channel ? sbg[v] : 1.0f));
+                    float u = acc[MT + mt][v] * (sa[mt] * (per_channel ? sbu[v] : 1.0f));
+                    // the unfused chain rounds both projections to 16 bits before the activation: do the same
+                    g = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(g)) : load16<HFRK_F16>(store16<HFRK_F16>(g));
+                    u = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(u)) : load16<HFRK_F16>(store16<HFRK_F16>(u));
+                    y[v] = silu_mul(g, u, inv_out_scale);
+                }
+                uint32_t packed = cvt_pk_fp8(y[0], y[1], 0u, false);
+                packed = cvt_pk_fp8(y[2], y[3], packed, true);
+                const bool live = mrow < a.m && n0 < n_out;
+                __builtin_amdgcn_raw_buffer_store_b32((int)packed, d_rsrc, live ? (int)((uint32_t)mrow * (uint32_t)n_out + (uint32_t)n0) : (int)kOutOfRange, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
@@ -167,7 +204,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         off[v] = (live && n0 + v < a.n) ? d_off + 2u * v : kOutOfRange;
-                        old[v] = a.accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(d_rsrc, (int)off[v], 0, 0) : 0u;
+                        old[v] = accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(base_rsrc, (int)off[v], 0, 0) : 0u;
                         sb[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, (live && per_channel && n0 + v < a.n) ? (n0 + v) * 4 : (int)kOutOfRange, 0, 0));
                     }
                 }
@@ -176,7 +213,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
                 for (int v = 0; v < 4; ++v) {
                     const float r = acc[rt * MT + mt][v] * (sa[mt] * (per_channel ? sb[v] : 1.0f));
                     const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)old[v]) : load16<HFRK_F16>((uint16_t)old[v]);
-                    const float sum = a.accumulate ? base + r : r;
+                    const float sum = accumulate ? base + r : r;
                     o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
                 }
                 if (vec) {
@@ -346,9 +383,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     }
 }
 
-template <int MA, int RT>
+template <int MA, int RT, bool SWIGLU>
 static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_stream_kernel<MA, RT>;
+    auto kern = skinny_gemm_stream_kernel<MA, RT, SWIGLU>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -361,23 +398,33 @@ static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t st
     return HFRK_SUCCESS;
 }
 
-int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream) {
+int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream) {
     if (lds_bytes != stream_lds_bytes(act_loads, row_tiles)) return HFRK_INVALID_CONFIG;
+    if (swiglu) {
+        if (row_tiles != 2) return HFRK_INVALID_CONFIG;
+        switch (act_loads) {
+            case 1: return launch_stream_one<1, 2, true>(args, lds_bytes, stream);
+            case 2: return launch_stream_one<2, 2, true>(args, lds_bytes, stream);
+            case 3: return launch_stream_one<3, 2, true>(args, lds_bytes, stream);
+            case 4: return launch_stream_one<4, 2, true>(args, lds_bytes, stream);
+        }
+        return HFRK_INVALID_CONFIG;
+    }
     if (row_tiles == 1) {
         switch (act_loads) {
-            case 1: return launch_stream_one<1, 1>(args, lds_bytes, stream);
-            case 2: return launch_stream_one<2, 1>(args, lds_bytes, stream);
-            case 3: return launch_stream_one<3, 1>(args, lds_bytes, stream);
-            case 4: return launch_stream_one<4, 1>(args, lds_bytes, stream);
+            case 1: return launch_stream_one<1, 1, false>(args, lds_bytes, stream);
+            case 2: return launch_stream_one<2, 1, false>(args, lds_bytes, stream);
+            case 3: return launch_stream_one<3, 1, false>(args, lds_bytes, stream);
+            case 4: return launch_stream_one<4, 1, false>(args, lds_bytes, stream);
         }
     } else if (row_tiles == 2) {
         switch (act_loads) {
-            case 3: return launch_stream_one<3, 2>(args, lds_bytes, stream);
-            case 4: return launch_stream_one<4, 2>(args, lds_bytes, stream);
-            case 5: return launch_stream_one<5, 2>(args, lds_bytes, stream);
-            case 6: return launch_stream_one<6, 2>(args, lds_bytes, stream);
-            case 7: return launch_stream_one<7, 2>(args, lds_bytes, stream);
-            case 8: return launch_stream_one<8, 2>(args, lds_bytes, stream);
+            case 3: return launch_stream_one<3, 2, false>(args, lds_bytes, stream);
+            case 4: return launch_stream_one<4, 2, false>(args, lds_bytes, stream);
+            case 5: return launch_stream_one<5, 2, false>(args, lds_bytes, stream);
+            case 6: return launch_stream_one<6, 2, false>(args, lds_bytes, stream);
+            case 7: return launch_stream_one<7, 2, false>(args, lds_bytes, stream);
+            case 8: return launch_stream_one<8, 2, false>(args, lds_bytes, stream);
         }
     }
     return HFRK_INVALID_CONFIG;

@@ -9,11 +9,6 @@
 
 namespace hfrk {
 
-__device__ __forceinline__ float silu_mul(float g, float u, float inv_scale) {
-    const float e = __builtin_amdgcn_exp2f(-g * 1.44269504089f);
-    return g * __builtin_amdgcn_rcpf(1.0f + e) * u * inv_scale;
-}
-
 // Zero rows*buffer_cols 16-bit elements, spread over every thread of the grid.
 __device__ __forceinline__ void zero_next_buffer(uint16_t* next_buffer, long total) {
     if (total <= 0) return;

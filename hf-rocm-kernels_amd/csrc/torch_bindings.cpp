@@ -171,6 +171,62 @@ int64_t skinny_gemm_scaled(at::Tensor& A, at::Tensor& B, at::Tensor& D, at::Tens
                                current_stream(A));
 }
 
+// The GEMM with the surrounding element-wise work folded in.  No reference counterpart as one op.
+//   epilogue 0: D = (base ? base : 0) + scale_a x scale_b x A.B, base a 16-bit [m,n] tensor (D itself, a residual) or None
+//   epilogue 1: B is a gate_up weight [k, 2*inter]; D fp8 [m, inter] = e4m3fn(silu(gate) * up / out_scale), the two
+//               projections rounded to `intermediate_dtype` (0 = float16, 1 = bfloat16) first
+int64_t skinny_gemm_fused(at::Tensor& A, at::Tensor& B, at::Tensor& D, const std::optional<at::Tensor>& base,
+                          at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
+                          int64_t epilogue, int64_t intermediate_dtype) {
+    TORCH_CHECK(A.dim() == 2 && A.is_contiguous(), "A must be a contiguous [m, k] tensor");
+    TORCH_CHECK(B.dim() == 2 && B.size(0) == A.size(1) && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
+    check_fp8(A, "A");
+    check_fp8(B, "B");
+    check_same_device(A, B, "B");
+    check_same_device(A, D, "D");
+    const int64_t m = A.size(0), n = B.size(1);
+    TORCH_CHECK(scale_a.scalar_type() == at::kFloat && scale_a.is_contiguous() && (scale_a.numel() == 1 || scale_a.numel() == m),
+                "scale_a must be float32 with 1 or m elements");
+    check_same_device(A, scale_a, "scale_a");
+    const float* scale_b_ptr = nullptr;  // None = 1
+    int sb_stride = 0;
+    if (scale_b.has_value()) {
+        TORCH_CHECK(scale_b->scalar_type() == at::kFloat && scale_b->is_contiguous() && (scale_b->numel() == 1 || scale_b->numel() == n),
+                    "scale_b must be float32 with 1 or n elements");
+        check_same_device(A, *scale_b, "scale_b");
+        scale_b_ptr = scale_b->data_ptr<float>();
+        sb_stride = scale_b->numel() == 1 ? 0 : 1;
+    }
+    int d_dtype;
+    const void* base_ptr = nullptr;
+    const float* out_scale_ptr = nullptr;
+    if (epilogue == HFRK_EPILOGUE_SWIGLU) {
+        TORCH_CHECK(n % 2 == 0 && D.dim() == 2 && D.size(0) == m && D.size(1) == n / 2 && D.is_contiguous(),
+                    "D must be a contiguous [m, n/2] tensor");
+        check_fp8(D, "D");
+        TORCH_CHECK(out_scale.has_value() && out_scale->numel() == 1 && out_scale->scalar_type() == at::kFloat,
+                    "out_scale must be one float32");
+        check_same_device(A, *out_scale, "out_scale");
+        TORCH_CHECK(!base.has_value(), "base cannot be combined with the SwiGLU epilogue");
+        TORCH_CHECK(intermediate_dtype == HFRK_F16 || intermediate_dtype == HFRK_BF16, "intermediate_dtype must be 0 (float16) or 1 (bfloat16)");
+        d_dtype = (int)intermediate_dtype;
+        out_scale_ptr = out_scale->data_ptr<float>();
+    } else {
+        TORCH_CHECK(D.dim() == 2 && D.size(0) == m && D.size(1) == n && D.is_contiguous(), "D must be a contiguous [m, n] tensor");
+        d_dtype = dtype16(D, "D");
+        if (base.has_value()) {
+            TORCH_CHECK(base->sizes() == D.sizes() && base->is_contiguous() && base->scalar_type() == D.scalar_type(),
+                        "base must be a contiguous tensor with D's shape and dtype");
+            check_same_device(A, *base, "base");
+            base_ptr = base->data_ptr();
+        }
+    }
+    DeviceScope scope(A);
+    return hfrk_skinny_gemm_fused(A.data_ptr(), B.data_ptr(), D.data_ptr(), base_ptr, scale_a.data_ptr<float>(),
+                                  scale_a.numel() == 1 ? 0 : 1, scale_b_ptr, sb_stride, out_scale_ptr, (int)m, (int)n, (int)A.size(1), (int)B.stride(1), d_dtype, (int)epilogue,
+                                  nullptr, current_stream(A));
+}
+
 }  // namespace
 
 TORCH_LIBRARY(_HFRK_C, ops) {
@@ -194,6 +250,11 @@ TORCH_LIBRARY(_HFRK_C, ops) {
 
     ops.def("skinny_gemm_scaled(Tensor A, Tensor B, Tensor! D, Tensor scale_a, Tensor scale_b, bool accumulate) -> int");
     ops.impl("skinny_gemm_scaled", c10::kCUDA, &skinny_gemm_scaled);
+
+    ops.def(
+        "skinny_gemm_fused(Tensor A, Tensor B, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
+        "Tensor? out_scale, int epilogue, int intermediate_dtype) -> int");
+    ops.impl("skinny_gemm_fused", c10::kCUDA, &skinny_gemm_fused);
 }
 
 // `import hf_rocm_kernels._HFRK_C` loads this library and thereby runs the registration above.

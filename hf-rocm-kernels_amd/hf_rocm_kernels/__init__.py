@@ -7,6 +7,7 @@ Importing this package loads both shared objects and fails if either is missing:
 from .operators.increment import increment
 from .operators.residual_rms import residual_rms
 from .operators.swiglu import swiglu
-from .operators.skinny_gemm import skinny_gemm, skinny_gemm_scaled
+from .operators.skinny_gemm import skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu
 
-__all__ = ["increment", "residual_rms", "swiglu", "skinny_gemm", "skinny_gemm_scaled"]
+__all__ = ["increment", "residual_rms", "swiglu", "skinny_gemm", "skinny_gemm_scaled", "skinny_gemm_add",
+           "skinny_gemm_swiglu"]

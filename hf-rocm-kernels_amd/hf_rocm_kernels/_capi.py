@@ -28,6 +28,10 @@ F16 = 0
 BF16 = 1
 FP8_E4M3FN = 2
 
+# enum hfrk_epilogue
+EPILOGUE_NONE = 0
+EPILOGUE_SWIGLU = 1
+
 GEMM_MAX_M = 64
 
 
@@ -52,6 +56,7 @@ SIGNATURES = {
     "hfrk_skinny_gemm_plan": (_i, [_i, _i, _i, ctypes.POINTER(GemmPlan)]),
     "hfrk_skinny_gemm": (_i, [_p, _p, _p, _p] + [_i] * 14 + [_p]),
     "hfrk_skinny_gemm_ex": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
+    "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_residual_rms": (_i, [_p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "hfrk_swiglu": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
 }

@@ -3,7 +3,7 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor
 
-from hf_rocm_kernels import residual_rms, skinny_gemm, swiglu
+from hf_rocm_kernels import residual_rms, skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu, swiglu
 
 
 def llama_mlp_combined_ops(
@@ -20,6 +20,7 @@ def llama_mlp_combined_ops(
     gate_up_gemm_hp: Tuple[Optional[int], Optional[int]] = (None, None),
     down_gemm_hp: Tuple[Optional[int], Optional[int]] = (None, None),
     add_residual: bool = False,
+    fused: bool = False,
 ) -> Tuple[Tensor, Tensor]:
     """Decoder MLP sub-block as four launches on one stream (reference: combined_ops/llama_mlp.py:7-60):
     residual RMSNorm -> fp8, gate_up GEMM, SwiGLU -> fp8, down GEMM.
@@ -32,9 +33,26 @@ def llama_mlp_combined_ops(
     - add_residual: the down projection accumulates onto a copy of the updated residual instead of zeros, so
       the first output is the block's output hidden state (residual + mlp) rounded once
 
+    - fused: three launches instead of four (plus a copy): the SwiGLU runs as the epilogue of the gate_up GEMM,
+      nothing is zeroed beforehand (the GEMMs overwrite), and with add_residual the down projection reads the
+      residual as its addend instead of accumulating onto a copy.  Same arithmetic, same roundings.
+
     RMSNorm and SwiGLU zero the buffer the following GEMM accumulates into, as in the reference.
     Returns (mlp_output, residual)."""
     del gate_up_gemm_hp, down_gemm_hp
+    if fused:
+        normalized, residual = residual_rms(input=attn_output, residual=residual, weight=rms_weight, epsilon=rms_epsilon,
+                                            scale_tensor=gate_up_input_scale)
+        swiglu_out = skinny_gemm_swiglu(normalized, gate_up_weight, gate_up_output_scale, None, down_input_scale,
+                                        intermediate_dtype=attn_output.dtype)
+        if add_residual:
+            mlp_output = skinny_gemm_add(swiglu_out, down_weight, down_output_scale, None, base=residual)
+        else:
+            mlp_output = torch.empty(size=(attn_output.size(0), down_weight.size(1)), dtype=attn_output.dtype,
+                                     device=attn_output.device)
+            skinny_gemm_scaled(swiglu_out, down_weight, down_output_scale,
+                               torch.ones(1, device=attn_output.device), output=mlp_output)
+        return mlp_output, residual
     m = attn_output.size(0)
     dtype = attn_output.dtype
 

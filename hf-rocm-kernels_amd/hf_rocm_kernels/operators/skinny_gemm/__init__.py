@@ -1,4 +1,5 @@
-from .wrapped import skinny_gemm, skinny_gemm_scaled
+from .wrapped import skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu
 from .data import generate_skinny_gemm_data, generate_llama_gemm_data
 
-__all__ = ["skinny_gemm", "skinny_gemm_scaled", "generate_skinny_gemm_data", "generate_llama_gemm_data"]
+__all__ = ["skinny_gemm", "skinny_gemm_scaled", "skinny_gemm_add", "skinny_gemm_swiglu", "generate_skinny_gemm_data",
+           "generate_llama_gemm_data"]

@@ -4,7 +4,7 @@ import torch
 from torch import Tensor
 
 from ... import _capi
-from .binding import _skinny_gemm, _skinny_gemm_scaled
+from .binding import _skinny_gemm, _skinny_gemm_fused, _skinny_gemm_scaled
 
 _OUT_DTYPES = (torch.bfloat16, torch.float16)
 
@@ -117,4 +117,90 @@ def skinny_gemm_scaled(
     status = _skinny_gemm_scaled(skinny_a, b, output, scale_a.contiguous().view(-1), scale_b.contiguous().view(-1),
                                  accumulate)
     _raise_on_status(status, "skinny_gemm_scaled")
+    return output
+
+
+class _ShapeOnly:
+    """Stands in for the (m, n) 16-bit tensor the fused op never materialises, for `skinny_gemm_checks`."""
+
+    def __init__(self, m: int, n: int, dtype: torch.dtype, device: torch.device):
+        self.shape, self.dtype, self.device = (m, n), dtype, device
+
+    def is_contiguous(self) -> bool:
+        return True
+
+    def stride(self) -> Tuple[int, int]:
+        return (self.shape[1], 1)
+
+
+def _scale_vectors(skinny_a: Tensor, b: Tensor, scale_a: Tensor, scale_b: Optional[Tensor]) -> Tuple[Tensor, Optional[Tensor]]:
+    m, n = skinny_a.size(0), b.size(1)
+    assert scale_a.numel() in (1, m) and scale_a.dtype == torch.float32, f"Expected 1 or {m} float32 in scale_a"
+    if scale_b is None:  # one combined scale in scale_a
+        return scale_a.contiguous().view(-1), None
+    assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
+    return scale_a.contiguous().view(-1), scale_b.contiguous().view(-1)
+
+
+def skinny_gemm_add(
+    skinny_a: Tensor,
+    b: Tensor,
+    scale_a: Tensor,
+    scale_b: Optional[Tensor],
+    base: Tensor,
+    output: Optional[Tensor] = None,
+) -> Tensor:
+    """output[i, j] = base[i, j] + scale_a[i] * scale_b[j] * (skinny_a @ b)[i, j], summed in fp32 and rounded once
+    (`scale_b` None = 1).
+    `base` has the output's shape and dtype (a residual stream, a bias broadcast beforehand); it is only read, so
+    the residual add after a projection costs no extra launch and no copy."""
+    m, n = skinny_a.size(0), b.size(1)
+    if output is None:
+        output = torch.empty(size=(m, n), dtype=base.dtype, device=skinny_a.device)
+    skinny_gemm_checks(skinny_a, b, scale_a.reshape(-1)[:1], output)
+    assert base.shape == output.shape and base.dtype == output.dtype and base.is_contiguous(), (
+        f"Expected base to be contiguous with {output.shape = } and {output.dtype = }")
+    sa, sb = _scale_vectors(skinny_a, b, scale_a, scale_b)
+    status = _skinny_gemm_fused(skinny_a, b, output, base, sa, sb, None, _capi.EPILOGUE_NONE, 0)
+    _raise_on_status(status, "skinny_gemm_fused")
+    return output
+
+
+def skinny_gemm_swiglu(
+    skinny_a: Tensor,
+    gate_up_weight: Tensor,
+    scale_a: Tensor,
+    scale_b: Optional[Tensor],
+    out_scale: Tensor,
+    output: Optional[Tensor] = None,
+    intermediate_dtype: torch.dtype = torch.bfloat16,
+) -> Tensor:
+    """gate_up projection and SwiGLU in one launch: with [gate | up] = scale_a * scale_b * (skinny_a @ gate_up_weight)
+    rounded to `intermediate_dtype`, returns float8_e4m3fn(silu(gate) * up / out_scale) of shape (m, n/2) -- what
+    `skinny_gemm` followed by `swiglu` produces, without the (m, n) intermediate and the second launch.
+    For m <= 16 and n % 32 == 0; other shapes run the two kernels."""
+    m, n = skinny_a.size(0), gate_up_weight.size(1)
+    assert n % 2 == 0, f"Expected an even number of gate_up columns but got {n}"
+    assert intermediate_dtype in _OUT_DTYPES, f"Expected one of {_OUT_DTYPES} but got {intermediate_dtype = }"
+    assert out_scale.numel() == 1 and out_scale.dtype == torch.float32, "Expected out_scale to be one float32"
+    if m > 16 or n % 32 != 0:
+        from ..swiglu import swiglu
+        gate_up = skinny_gemm_scaled(skinny_a, gate_up_weight, scale_a,
+                                     scale_b if scale_b is not None else torch.ones(1, device=skinny_a.device),
+                                     output=torch.empty((m, n), dtype=intermediate_dtype, device=skinny_a.device))
+        result = swiglu(gate_up_proj=gate_up, scale_tensor=out_scale)
+        if output is None:
+            return result
+        output.copy_(result)
+        return output
+    if output is None:
+        output = torch.empty(size=(m, n // 2), dtype=torch.float8_e4m3fn, device=skinny_a.device)
+    assert output.shape == (m, n // 2) and output.dtype == torch.float8_e4m3fn and output.is_contiguous(), (
+        f"Expected a contiguous float8_e4m3fn output of shape {(m, n // 2)}")
+    skinny_gemm_checks(skinny_a, gate_up_weight, scale_a.reshape(-1)[:1],
+                       _ShapeOnly(m, n, intermediate_dtype, skinny_a.device))
+    sa, sb = _scale_vectors(skinny_a, gate_up_weight, scale_a, scale_b)
+    status = _skinny_gemm_fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU,
+                                _capi.BF16 if intermediate_dtype == torch.bfloat16 else _capi.F16)
+    _raise_on_status(status, "skinny_gemm_fused")
     return output

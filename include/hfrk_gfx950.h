@@ -40,6 +40,9 @@ enum hfrk_status {
 /* Element types of 16-bit tensors. */
 enum hfrk_dtype { HFRK_F16 = 0, HFRK_BF16 = 1, HFRK_FP8_E4M3FN = 2 };
 
+/* What happens to the product before it is stored (hfrk_skinny_gemm_fused). */
+enum hfrk_epilogue { HFRK_EPILOGUE_NONE = 0, HFRK_EPILOGUE_SWIGLU = 1 };
+
 /* Largest m the skinny GEMM accepts. */
 #define HFRK_GEMM_MAX_M 64
 
@@ -105,6 +108,21 @@ int hfrk_skinny_gemm(const void* A, const void* B, void* D, const float* scale_t
 int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
                         const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
                         int accumulate, const hfrk_gemm_plan* plan, void* stream);
+
+/* The GEMM with what the decoder block does around it folded in (no reference counterpart as one call; it stands
+ * for skinny_gemm followed by swiglu in hf_rocm_kernels/combined_ops/llama_mlp.py:43-56, and for the residual add
+ * after the down projection).
+ *   epilogue HFRK_EPILOGUE_NONE:   D[i,j] = (base ? base[i,j] : 0) + scale_a[i] * scale_b[j] * sum_k A[i,k] B[k,j]
+ *       base: 16-bit [m,n] like D, may be D itself (= accumulate) or another tensor (e.g. the residual), or NULL.
+ *   epilogue HFRK_EPILOGUE_SWIGLU: B is a gate_up weight, gate rows [0, n/2), up rows [n/2, n);
+ *       D[i,j] = e4m3fn( silu(g) * u / out_scale[0] ),  g, u = the two projections of column j, each rounded to
+ *       d_dtype first (what the unfused chain stores between its two kernels);  D is fp8 [m, n/2], 4-byte aligned.
+ *       Needs m <= 16, n % 32 == 0, base == NULL; otherwise HFRK_BAD_SHAPE (callers then run the two kernels).
+ * Scales and plan as in hfrk_skinny_gemm_ex; a plan passed with the SwiGLU epilogue describes n/2 output columns
+ * with wk = 2. */
+int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
+                           const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k,
+                           int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
 
 /* residual <- input + residual (one 16-bit add); output <- rmsnorm(residual) * weight, optionally / scale -> fp8.
  * Replaces `void residual_rms(...)` at csrc/op_src/residual_rms/residual_rms_dispatch.cu:8-63.

@@ -255,3 +255,112 @@ def test_capturable_in_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+# ---- fused forms: residual addend and SwiGLU epilogue -----------------------------------------------------------------
+
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 14336), (8, 4096, 4096), (16, 1040, 1024), (13, 130, 512), (32, 4096, 4096),
+                                   (64, 1000, 2048)])
+def test_base_addend_is_read_not_written(m, n, k):
+    """D = base + scale * A.B with base a separate tensor: one fp32 sum, one rounding; base stays untouched."""
+    from hf_rocm_kernels import skinny_gemm_add
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=31)
+    base = torch.randn(m, n, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).cuda()
+    keep = base.clone()
+    out = skinny_gemm_add(a, b, sa, sw, base)
+    assert torch.equal(base, keep)
+    check_against_oracle(out, a, b, sa, sw, base=keep)
+    # in place (base is the output) gives the same bits
+    again = skinny_gemm_add(a, b, sa, sw, base, output=base)
+    assert again.data_ptr() == base.data_ptr() and torch.equal(again, out)
+
+
+def _swiglu_oracle(a, w, sa, sb, out_scale, dtype):
+    """(fp8 result of the oracle chain, tolerance in fp8 units).  Two correct GEMMs may round a 16-bit projection
+    differently: each lies within `error_bound` (1 ulp + 2^-16 sum|a b|) of the exact product, so gate and up can
+    differ by twice that, which moves silu(gate) * up by at most 1.1 |up| dgate + |silu(gate)| dup (|silu'| <= 1.1);
+    on top of that the fp8 rounding may flip by one step."""
+    og = _oracle()
+    from oracle import swiglu as osw
+    a_c, w_c, sa_c, sb_c = a.cpu(), w.cpu(), sa.cpu(), sb.cpu()
+    gate_up = og.reference_skinny_gemm(a_c, w_c, sa_c, sb_c, out_dtype=dtype)
+    ref = osw.reference_swiglu(gate_up, out_scale.cpu())
+    exact = og.exact_skinny_gemm(a_c, w_c, sa_c, sb_c)
+    bound = og.error_bound(a_c, w_c, sa_c, sb_c, dtype, exact)
+    half = exact.shape[1] // 2
+    g, u = exact[:, :half], exact[:, half:]
+    dg, du = 2 * bound[:, :half], 2 * bound[:, half:]
+    silu = g / (1 + torch.exp(-g))
+    moved = (1.1 * u.abs() * dg + silu.abs() * du + 1.1 * dg * du) / float(out_scale)
+    step = torch.maximum(ref.float().abs() * 2.0 ** -3, torch.tensor(2.0 ** -9))
+    return ref, (step + moved).float()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("per_channel", [False, True])
+@pytest.mark.parametrize("m,n,k", [(1, 512, 1024), (5, 2080, 512), (8, 28672, 4096), (13, 1024, 2048), (16, 28672, 4096),
+                                   (16, 64, 256)])
+def test_swiglu_epilogue_matches_the_two_kernel_chain(m, n, k, per_channel, dtype):
+    """One launch (GEMM with SwiGLU epilogue) against GEMM -> 16-bit -> swiglu, on the device and in the oracle.
+    The two device paths may sum K in a different order, so a 16-bit projection can differ by one rounding and an
+    fp8 output by one step; such flips must be rare and never larger."""
+    from hf_rocm_kernels import skinny_gemm_scaled, skinny_gemm_swiglu, swiglu
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    a, w, sa, sw = generate_llama_gemm_data(m, n, k, seed=40 + m, per_token=(m > 4), per_channel=per_channel, weight_std=0.05)
+    out_scale = torch.tensor([8.0 / 448], dtype=torch.float32).cuda()
+    fused = skinny_gemm_swiglu(a, w, sa, sw, out_scale, intermediate_dtype=dtype)
+    assert fused.dtype == torch.float8_e4m3fn and fused.shape == (m, n // 2)
+    gate_up = skinny_gemm_scaled(a, w, sa, sw, output=torch.empty(m, n, dtype=dtype).cuda())
+    chain = swiglu(gate_up, out_scale)
+    ref, tol = _swiglu_oracle(a, w, sa, sw, out_scale, dtype)
+    f = fused.cpu().float()
+    assert not f.isnan().any()
+    for name, other in (("device chain", chain.cpu().float()), ("oracle", ref.float())):
+        d = (f - other).abs()
+        assert (d <= tol).all(), (name, float((d / tol).max()))
+        assert (d > 0).float().mean() < 0.02, (name, float((d > 0).float().mean()))
+
+
+def test_swiglu_epilogue_limits_and_fallback():
+    from hf_rocm_kernels import _capi, skinny_gemm_swiglu
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    lib = _capi.load()
+    a, w, sa, sw = generate_llama_gemm_data(17, 512, 512, seed=3)
+    out_scale = torch.ones(1).cuda()
+    out = torch.empty(17, 256, dtype=torch.float8_e4m3fn).cuda()
+    args = lambda m, n: (a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                         out_scale.data_ptr(), m, n, 512, 512, _capi.BF16, _capi.EPILOGUE_SWIGLU, None, None)
+    assert lib.hfrk_skinny_gemm_fused(*args(17, 512)) == _capi.BAD_SHAPE      # m > 16: callers run the two kernels
+    assert lib.hfrk_skinny_gemm_fused(*args(8, 496)) == _capi.BAD_SHAPE       # n % 32 != 0
+    bad = list(args(8, 512)); bad[3] = out.data_ptr()
+    assert lib.hfrk_skinny_gemm_fused(*bad) == _capi.BAD_SHAPE                # base with the SwiGLU epilogue
+    bad = list(args(8, 512)); bad[14] = 7
+    assert lib.hfrk_skinny_gemm_fused(*bad) == _capi.INVALID_CONFIG
+    # the Python wrapper falls back to GEMM + swiglu above 16 rows
+    got = skinny_gemm_swiglu(a, w, sa, sw, out_scale)
+    ref, tol = _swiglu_oracle(a, w, sa, sw, out_scale, torch.bfloat16)
+    assert ((got.cpu().float() - ref.float()).abs() <= tol).all()
+
+
+@pytest.mark.parametrize("m,n,k", [(8, 1024, 2048), (16, 6144, 1024), (3, 2080 * 2, 512)])
+def test_swiglu_epilogue_under_every_split(m, n, k):
+    """Forced plans: grids that cut (gate, up) tile pairs between waves and between workgroups in different places."""
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    lib = _capi.load()
+    a, w, sa, sw = generate_llama_gemm_data(m, n, k, seed=77, weight_std=0.05)
+    out_scale = torch.tensor([8.0 / 448], dtype=torch.float32).cuda()
+    ref, tol = _swiglu_oracle(a, w, sa, sw, out_scale, torch.bfloat16)
+    ma, kc, groups = (m + 3) // 4, k // 256, (n // 2) // 16
+    for grid in sorted({min(g, groups * kc) for g in (256, 200, 64, 7, 1)}):
+        plan = _capi.GemmPlan((ma + 3) // 4, 0, 2, ma, grid, groups, kc, 8 * (2 + (ma + 3) // 4) * 4096)
+        out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
+        st = lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                                        out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
+                                        ctypes.byref(plan), torch.cuda.current_stream().cuda_stream)
+        assert st == 0, (grid, st)
+        torch.cuda.synchronize()
+        f = out.cpu().float()
+        assert not f.isnan().any(), grid
+        assert ((f - ref.float()).abs() <= tol).all(), grid

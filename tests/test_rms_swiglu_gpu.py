@@ -128,9 +128,10 @@ def test_rms_rejects_bad_epsilon_and_mixed_dtypes():
         residual_rms(x, x.clone(), w.to(torch.bfloat16), 1e-5)
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("add_residual", [False, True])
 @pytest.mark.parametrize("m", [1, 8, 16])
-def test_llama_mlp_chain(m, add_residual):
+def test_llama_mlp_chain(m, add_residual, fused):
     """BASELINE config 4: hidden 4096, gate_up 28672x4096, down 4096x14336, eps 1e-5, weight ~ 1+N(0,0.1), bf16."""
     from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
     from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
@@ -153,7 +154,7 @@ def test_llama_mlp_chain(m, add_residual):
     loose_out, _ = omlp.reference_llama_mlp(*cpu_args, add_residual=add_residual, exact_norm=False)
     dev = [t.cuda() if isinstance(t, torch.Tensor) else t for t in args_cpu]
     dev[4], dev[7] = wgu8.cuda().t(), wd8.cuda().t()
-    out, res = llama_mlp_combined_ops(*dev, add_residual=add_residual)
+    out, res = llama_mlp_combined_ops(*dev, add_residual=add_residual, fused=fused)
     assert torch.equal(res.cpu().view(torch.int16), ref_res.view(torch.int16))
     # Against the chain whose normalisation rounds once (what the kernel computes): the chain quantises twice on the
     # way, so a rare fp8 boundary flip upstream moves a down-projection output by more than the single-GEMM bound;
