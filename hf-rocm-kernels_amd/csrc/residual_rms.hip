@@ -58,8 +58,17 @@ __global__ void __launch_bounds__(kRmsMaxThreads) residual_rms_vec_kernel(
     __shared__ float red[16];
     const long row_off = (long)blockIdx.x * cols;
     const int nvec = cols >> 3;
-    uint4 z[ITERS];
+    uint4 z[ITERS], wreg[ITERS];
     float ssq = 0.f;
+    // Everything the second pass needs is requested now, so that the kernel pays one memory latency, not two.
+    float scale = 1.f;
+    if constexpr (FP8_OUT) scale = scale_tensor[0];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = threadIdx.x + it * blockDim.x;
+        wreg[it] = make_uint4(0, 0, 0, 0);
+        if (v < nvec) wreg[it] = reinterpret_cast<const uint4*>(weight)[v];
+    }
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int v = threadIdx.x + it * blockDim.x;
@@ -83,14 +92,13 @@ __global__ void __launch_bounds__(kRmsMaxThreads) residual_rms_vec_kernel(
     }
     const float total = block_sum(ssq, red);
     const float norm = rsqrtf(total / (float)cols + epsilon);
-    float inv_scale = 1.f;
-    if constexpr (FP8_OUT) inv_scale = 1.f / scale_tensor[0];
+    const float inv_scale = 1.f / scale;
 
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int v = threadIdx.x + it * blockDim.x;
         if (v < nvec) {
-            const uint4 w = reinterpret_cast<const uint4*>(weight)[v];
+            const uint4 w = wreg[it];
             const uint32_t zw[4] = {z[it].x, z[it].y, z[it].z, z[it].w}, ww[4] = {w.x, w.y, w.z, w.w};
             if constexpr (FP8_OUT) {
                 float y[8];

@@ -31,16 +31,27 @@ __global__ void __launch_bounds__(1024) swiglu_vec_kernel(const uint16_t* __rest
                                                           int rows, int cols, int buffer_cols) {
     const int vpr = cols >> 3;  // 8-element pieces per output row
     const long nvec = (long)rows * vpr;
+    const long stride = (long)gridDim.x * blockDim.x;
+    long v = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    v4i g = {0, 0, 0, 0}, u = {0, 0, 0, 0};
+    auto fetch = [&](long idx) __attribute__((always_inline)) {
+        const long r = idx / vpr;
+        const int c = (int)(idx - r * vpr);
+        const uint16_t* const grow = gate_up + r * 2 * cols;
+        g = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(grow) + c);
+        u = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(grow + cols) + c);
+    };
+    // The first piece is requested before the scale, and each next piece before the current one is processed: the
+    // kernel is a few microseconds long and pays every dependent memory latency in full.
+    if (v < nvec) fetch(v);
     const float s = scale_tensor[0];
     const float inv_scale = (s != 0.f) ? 1.f / s : 1.f;
-    for (long v = (long)blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += (long)gridDim.x * blockDim.x) {
-        const long r = v / vpr;
-        const int c = (int)(v - r * vpr);
-        const uint16_t* const grow = gate_up + r * 2 * cols;
-        const v4i g = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(grow) + c);
-        const v4i u = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(grow + cols) + c);
+    while (v < nvec) {
         const uint32_t gw[4] = {(uint32_t)g[0], (uint32_t)g[1], (uint32_t)g[2], (uint32_t)g[3]};
         const uint32_t uw[4] = {(uint32_t)u[0], (uint32_t)u[1], (uint32_t)u[2], (uint32_t)u[3]};
+        const long cur = v;
+        v += stride;
+        if (v < nvec) fetch(v);
         float y[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -51,6 +62,8 @@ __global__ void __launch_bounds__(1024) swiglu_vec_kernel(const uint16_t* __rest
         p0 = cvt_pk_fp8(y[2], y[3], p0, true);
         uint32_t p1 = cvt_pk_fp8(y[4], y[5], 0u, false);
         p1 = cvt_pk_fp8(y[6], y[7], p1, true);
+        const long r = cur / vpr;
+        const int c = (int)(cur - r * vpr);
         reinterpret_cast<uint2*>(output + r * cols)[c] = make_uint2(p0, p1);
     }
     zero_next_buffer(next_buffer, (long)rows * buffer_cols);
