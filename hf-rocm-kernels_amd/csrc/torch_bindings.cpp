@@ -171,6 +171,68 @@ int64_t skinny_gemm_scaled(at::Tensor& A, at::Tensor& B, at::Tensor& D, at::Tens
                                current_stream(A));
 }
 
+static void next_buffer_args(const at::Tensor& like, const at::Tensor& next_buffer, int64_t rows, void** nb, int64_t* buffer_cols) {
+    *nb = nullptr;
+    *buffer_cols = 0;
+    if (next_buffer.numel() > 0) {
+        TORCH_CHECK(next_buffer.dim() == 2 && next_buffer.size(0) == rows && next_buffer.is_contiguous(),
+                    "next_buffer must be a contiguous [rows, buffer_cols] tensor");
+        TORCH_CHECK(next_buffer.element_size() == 2, "next_buffer must hold 16-bit elements");
+        check_same_device(like, next_buffer, "next_buffer");
+        *buffer_cols = next_buffer.size(1);
+        *nb = next_buffer.data_ptr();
+    }
+}
+
+// residual RMSNorm with per-row dynamic fp8 quantisation: output fp8 [rows, cols], scales fp32 [rows].  No reference counterpart.
+void residual_rms_dynamic(at::Tensor& input, at::Tensor& residual, at::Tensor& weight, double epsilon, at::Tensor& output,
+                          at::Tensor& scales, at::Tensor& next_buffer) {
+    TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous [rows, cols] tensor");
+    TORCH_CHECK(residual.sizes() == input.sizes() && residual.is_contiguous(), "residual must match input and be contiguous");
+    TORCH_CHECK(weight.dim() == 1 && weight.size(0) == input.size(1) && weight.is_contiguous(), "weight must be [cols]");
+    TORCH_CHECK(output.sizes() == input.sizes() && output.is_contiguous(), "output must match input and be contiguous");
+    const int io = dtype16(input, "input");
+    TORCH_CHECK(residual.scalar_type() == input.scalar_type() && weight.scalar_type() == input.scalar_type(),
+                "input, residual and weight must share one 16-bit dtype");
+    check_fp8(output, "output");
+    TORCH_CHECK(scales.scalar_type() == at::kFloat && scales.is_contiguous() && scales.numel() == input.size(0),
+                "scales must be a contiguous float32 tensor with one element per row");
+    check_same_device(input, residual, "residual");
+    check_same_device(input, weight, "weight");
+    check_same_device(input, output, "output");
+    check_same_device(input, scales, "scales");
+    void* nb;
+    int64_t buffer_cols;
+    next_buffer_args(input, next_buffer, input.size(0), &nb, &buffer_cols);
+    DeviceScope scope(input);
+    raise_on(hfrk_residual_rms_dynamic(input.data_ptr(), residual.data_ptr(), weight.data_ptr(), (float)epsilon, output.data_ptr(),
+                                       scales.data_ptr<float>(), nb, (int)input.size(0), (int)input.size(1), (int)buffer_cols, io,
+                                       current_stream(input)),
+             "residual_rms_dynamic");
+}
+
+// SwiGLU with per-row dynamic fp8 quantisation.  No reference counterpart.
+void swiglu_dynamic(at::Tensor& gate_up, at::Tensor& output, at::Tensor& scales, at::Tensor& next_buffer) {
+    TORCH_CHECK(gate_up.dim() == 2 && gate_up.is_contiguous() && gate_up.size(1) % 2 == 0,
+                "gate_up must be a contiguous [rows, 2*cols] tensor");
+    const int io = dtype16(gate_up, "gate_up");
+    const int64_t rows = gate_up.size(0), cols = gate_up.size(1) / 2;
+    check_fp8(output, "output");
+    TORCH_CHECK(output.dim() == 2 && output.size(0) == rows && output.size(1) == cols && output.is_contiguous(),
+                "output must be a contiguous [rows, cols] tensor");
+    TORCH_CHECK(scales.scalar_type() == at::kFloat && scales.is_contiguous() && scales.numel() == rows,
+                "scales must be a contiguous float32 tensor with one element per row");
+    check_same_device(gate_up, output, "output");
+    check_same_device(gate_up, scales, "scales");
+    void* nb;
+    int64_t buffer_cols;
+    next_buffer_args(gate_up, next_buffer, rows, &nb, &buffer_cols);
+    DeviceScope scope(gate_up);
+    raise_on(hfrk_swiglu_dynamic(gate_up.data_ptr(), output.data_ptr(), scales.data_ptr<float>(), nb, (int)rows, (int)cols,
+                                 (int)buffer_cols, io, current_stream(gate_up)),
+             "swiglu_dynamic");
+}
+
 // The GEMM with the surrounding element-wise work folded in.  No reference counterpart as one op.
 //   epilogue 0: D = (base ? base : 0) + scale_a x scale_b x A.B, base a 16-bit [m,n] tensor (D itself, a residual) or None
 //   epilogue 1: B is a gate_up weight [k, 2*inter]; D fp8 [m, inter] = e4m3fn(silu(gate) * up / out_scale), the two
@@ -255,6 +317,14 @@ TORCH_LIBRARY(_HFRK_C, ops) {
         "skinny_gemm_fused(Tensor A, Tensor B, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
         "Tensor? out_scale, int epilogue, int intermediate_dtype) -> int");
     ops.impl("skinny_gemm_fused", c10::kCUDA, &skinny_gemm_fused);
+
+    ops.def(
+        "residual_rms_dynamic(Tensor input, Tensor! residual, Tensor weight, float epsilon, Tensor! output, "
+        "Tensor! scales, Tensor! next_buffer) -> ()");
+    ops.impl("residual_rms_dynamic", c10::kCUDA, &residual_rms_dynamic);
+
+    ops.def("swiglu_dynamic(Tensor gate_up, Tensor! output, Tensor! scales, Tensor! next_buffer) -> ()");
+    ops.impl("swiglu_dynamic", c10::kCUDA, &swiglu_dynamic);
 }
 
 // `import hf_rocm_kernels._HFRK_C` loads this library and thereby runs the registration above.

@@ -5,9 +5,9 @@ Same names as the reference package (hf_rocm_kernels/__init__.py:1-6): four oper
 Importing this package loads both shared objects and fails if either is missing: there is no fallback path.
 """
 from .operators.increment import increment
-from .operators.residual_rms import residual_rms
-from .operators.swiglu import swiglu
+from .operators.residual_rms import residual_rms, residual_rms_dynamic
+from .operators.swiglu import swiglu, swiglu_dynamic
 from .operators.skinny_gemm import skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu
 
 __all__ = ["increment", "residual_rms", "swiglu", "skinny_gemm", "skinny_gemm_scaled", "skinny_gemm_add",
-           "skinny_gemm_swiglu"]
+           "skinny_gemm_swiglu", "residual_rms_dynamic", "swiglu_dynamic"]

@@ -59,6 +59,8 @@ SIGNATURES = {
     "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_residual_rms": (_i, [_p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "hfrk_swiglu": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "hfrk_residual_rms_dynamic": (_i, [_p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "hfrk_swiglu_dynamic": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
 }
 
 _lib = None

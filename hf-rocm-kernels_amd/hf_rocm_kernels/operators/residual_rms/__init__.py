@@ -1,4 +1,4 @@
-from .wrapped import residual_rms
+from .wrapped import residual_rms, residual_rms_dynamic
 from .data import generate_residual_rms_data
 
-__all__ = ["residual_rms", "generate_residual_rms_data"]
+__all__ = ["residual_rms", "residual_rms_dynamic", "generate_residual_rms_data"]

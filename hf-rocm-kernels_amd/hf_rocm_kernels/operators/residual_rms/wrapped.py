@@ -99,3 +99,24 @@ def residual_rms(
         force_scalar=force_scalar,
     )
     return output, residual
+
+
+def residual_rms_dynamic(
+    input: Tensor,
+    residual: Tensor,
+    weight: Tensor,
+    epsilon: float,
+    next_buffer: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """residual <- input + residual, RMS normalisation, and per-row dynamic quantisation to float8_e4m3fn: every row
+    gets its own scale amax/448, so no activation scale has to be known in advance.
+    Returns (output fp8 (rows, cols), residual, scales fp32 (rows,)); `scales` is the GEMM's per-token `scale_a`.
+    Rows must be 16-byte aligned (cols % 8 == 0) and at most 32768 wide."""
+    if next_buffer is None:
+        next_buffer = torch.empty(size=(input.size(0), 0), device=input.device, dtype=input.dtype)
+    residual_rms_checks(input, residual, weight, None, epsilon, next_buffer)
+    assert input.size(1) % 8 == 0 and input.size(1) <= 32768, f"Expected cols % 8 == 0 and cols <= 32768: {input.shape = }"
+    output = torch.empty(size=input.shape, dtype=torch.float8_e4m3fn, device=input.device)
+    scales = torch.empty(size=(input.size(0),), dtype=torch.float32, device=input.device)
+    torch.ops._HFRK_C.residual_rms_dynamic(input, residual, weight, epsilon, output, scales, next_buffer)
+    return output, residual, scales

@@ -1,4 +1,4 @@
-from .wrapped import swiglu
+from .wrapped import swiglu, swiglu_dynamic
 from .data import generate_swiglu_data
 
-__all__ = ["swiglu", "generate_swiglu_data"]
+__all__ = ["swiglu", "swiglu_dynamic", "generate_swiglu_data"]

@@ -141,6 +141,19 @@ int hfrk_residual_rms(const void* input, void* residual, const void* weight, con
 int hfrk_swiglu(const void* gate_up, const float* scale_tensor, void* output, void* next_buffer, int rows,
                 int cols, int buffer_cols, int io_dtype, int num_threads, int force_scalar, void* stream);
 
+/* Per-token dynamic quantisation (no reference counterpart: the reference's kernels take one static scale_tensor,
+ * hf_rocm_kernels/operators/residual_rms/wrapped.py:94-95, operators/swiglu/wrapped.py:49-84).
+ *   residual <- input + residual;  y = rmsnorm(residual) * weight       (hfrk_residual_rms_dynamic)
+ *   y = silu(gate_up[:, :cols]) * gate_up[:, cols:]                     (hfrk_swiglu_dynamic)
+ *   scales[r] = max(amax_c |y[r,c]| / 448, FLT_MIN);  output[r,c] = e4m3fn(y[r,c] / scales[r])
+ * scales: rows fp32 values, ready to be the GEMM's per-token scale_a.  Rows must be 16-byte aligned (cols % 8 == 0)
+ * and cols <= 32768, else HFRK_BAD_SHAPE / HFRK_BAD_ALIGNMENT.  next_buffer as in hfrk_residual_rms. */
+int hfrk_residual_rms_dynamic(const void* input, void* residual, const void* weight, float epsilon, void* output,
+                              float* scales, void* next_buffer, int rows, int cols, int buffer_cols, int io_dtype,
+                              void* stream);
+int hfrk_swiglu_dynamic(const void* gate_up, void* output, float* scales, void* next_buffer, int rows, int cols,
+                        int buffer_cols, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -50,3 +50,19 @@ def precise_residual_rms(input: torch.Tensor, residual: torch.Tensor, weight: to
     else:
         out = normed
     return out, x
+
+
+def precise_residual_rms_dynamic(input: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, epsilon: float
+                                 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Per-row dynamic quantisation of the normalised row (no reference counterpart; the reference's
+    operators/residual_rms/reference.py:7-36 quantises with one static scale): the residual is the 16-bit sum as in
+    `reference_residual_rms`, y = weight * z * rsqrt(mean(z^2) + eps) in float64, scale[row] = amax|y| / 448 rounded to
+    float32, output = e4m3fn(y / scale).  Returns (output fp8, new residual (16-bit), scales fp32 [rows], y float64).
+    Pinned by the textbook formula and by what the scaling fixes: every non-zero row of the output has a code of
+    magnitude 448, and output * scale reproduces y to within half an fp8 step."""
+    z = (input.float() + residual.float()).to(input.dtype)
+    x = z.to(torch.float64)
+    y = weight.to(torch.float64) * x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + epsilon)
+    scales = fp8.amax_scale(y, dim=1)
+    out, _ = fp8.fp8_quantize(y, scales)
+    return out, z, scales.reshape(-1), y

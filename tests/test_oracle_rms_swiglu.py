@@ -144,3 +144,38 @@ def test_mlp_chain_is_the_composition_of_its_parts():
     out_res, _ = omlp.reference_llama_mlp(x, r, w, 1e-5, wgu8, in_gu, in_gu * s_gu, wd8, in_d, in_d * s_d, add_residual=True)
     manual = (og.reference_skinny_gemm(a8, wd8, in_d * s_d, one, out_dtype=torch.float32) + res2.float()).to(dtype)
     assert torch.equal(out_res, manual)
+
+
+# ---- per-row dynamic quantisation (oracle of the *_dynamic operators) ----------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dynamic_quantisation_oracles_are_fixed_by_their_scaling(dtype):
+    """What the definition forces: the row maximum lands on +-448 exactly, the scale is amax/448, and dequantising
+    reproduces y to within half an fp8 step (relative 2^-4 for normals, 2^-10 absolute in code units below)."""
+    from oracle import residual_rms as orms
+    from oracle import swiglu as osw
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(6, 512, generator=g).to(dtype)
+    r = torch.randn(6, 512, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(512, generator=g)).to(dtype)
+    q, z, scales, y = orms.precise_residual_rms_dynamic(x, r, w, 1e-5)
+    assert torch.equal(z, (x.float() + r.float()).to(dtype))
+    gu = torch.randn(5, 2 * 384, generator=g).mul(3)
+    gu[1] *= 8.0  # an outlier row gets its own scale
+    gu = gu.to(dtype)
+    q2, scales2, y2 = osw.precise_swiglu_dynamic(gu)
+    for qq, ss, yy in ((q, scales, y), (q2, scales2, y2)):
+        assert ss.dtype == torch.float32 and ss.shape == (yy.shape[0],)
+        assert torch.allclose(ss.double(), yy.abs().amax(dim=1) / 448.0, rtol=1e-6)
+        assert (qq.float().abs().amax(dim=1) == 448.0).all()
+        deq = qq.double() * ss.double()[:, None]
+        half_step = torch.maximum(yy.abs() * 2.0 ** -4, ss.double()[:, None] * 2.0 ** -10)
+        assert ((deq - yy).abs() <= half_step * 1.0001).all()
+    # rows scale independently: the outlier row does not cost the others their resolution
+    assert scales2[1] > 10 * scales2[0]
+    # textbook check of y against plain float64 arithmetic written out
+    zz = z.double()
+    manual = w.double() * zz / torch.sqrt((zz * zz).mean(dim=1, keepdim=True) + 1e-5)
+    assert torch.allclose(y, manual, rtol=1e-12, atol=0)
+    gate, up = gu[:, :384].double(), gu[:, 384:].double()
+    assert torch.allclose(y2, gate / (1 + torch.exp(-gate)) * up, rtol=1e-12, atol=1e-300)

@@ -168,3 +168,87 @@ def test_llama_mlp_chain(m, add_residual, fused):
     # agreement at the level those flips allow, a few percent of the output's spread
     dl = (o - loose_out.float()).abs()
     assert float(dl.mean()) < 0.03 * float(loose_out.float().std()) + 1e-2
+
+
+# ---- per-row dynamic quantisation ----------------------------------------------------------------------------------------
+
+def _check_dynamic(q_dev, scales_dev, q_ref, scales_ref, y):
+    s_dev, s_ref = scales_dev.cpu().double(), scales_ref.double()
+    assert ((s_dev - s_ref).abs() <= 4e-6 * s_ref).all(), float(((s_dev - s_ref).abs() / s_ref).max())
+    qd = q_dev.cpu().float()
+    assert not qd.isnan().any()
+    nonzero = y.abs().amax(dim=1) > 0
+    assert (qd.abs().amax(dim=1)[nonzero] == 448.0).all()
+    d = (qd - q_ref.float()).abs()
+    step = torch.maximum(q_ref.float().abs() * 2.0 ** -3, torch.tensor(2.0 ** -9))
+    assert (d <= step).all()
+    assert (d > 0).float().mean() < 0.01, float((d > 0).float().mean())
+    # in real units: dequantised values reproduce y to half an fp8 step (plus the fp32 evaluation of y itself)
+    deq = q_dev.cpu().double() * s_dev[:, None]
+    assert ((deq - y).abs() <= y.abs() * (2.0 ** -4 + 1e-5) + s_dev[:, None] * 2.0 ** -10 * 1.001).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (8, 4096), (16, 8192), (5, 1024), (3, 32768), (7, 64), (64, 14336)])
+def test_residual_rms_dynamic(rows, cols, dtype):
+    from hf_rocm_kernels import residual_rms_dynamic
+    from oracle import residual_rms as orms
+    g = torch.Generator().manual_seed(rows * 100 + cols)
+    x = torch.randn(rows, cols, generator=g).to(dtype)
+    r = torch.randn(rows, cols, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    if rows > 2:
+        x[1] *= 25.0
+    q_ref, z_ref, s_ref, y = orms.precise_residual_rms_dynamic(x, r, w, 1e-5)
+    nb = torch.full((rows, 24), 7.0, dtype=dtype).cuda()
+    q, res, scales = residual_rms_dynamic(x.cuda(), r.cuda(), w.cuda(), 1e-5, next_buffer=nb)
+    assert torch.equal(res.cpu().view(torch.int16), z_ref.view(torch.int16))
+    assert (nb == 0).all()
+    _check_dynamic(q, scales, q_ref, s_ref, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(1, 14336), (8, 14336), (16, 28672), (5, 256), (3, 32768), (7, 8)])
+def test_swiglu_dynamic(rows, cols, dtype):
+    from hf_rocm_kernels import swiglu_dynamic
+    from oracle import swiglu as osw
+    g = torch.Generator().manual_seed(rows * 100 + cols + 1)
+    gu = torch.randn(rows, 2 * cols, generator=g).mul(2.5).to(dtype)
+    q_ref, s_ref, y = osw.precise_swiglu_dynamic(gu)
+    q, scales = swiglu_dynamic(gu.cuda())
+    _check_dynamic(q, scales, q_ref, s_ref, y)
+
+
+def test_dynamic_scales_feed_the_gemm():
+    """rms_dynamic -> per-token GEMM: the device's own fp8 rows and scales through the GEMM oracle."""
+    from hf_rocm_kernels import residual_rms_dynamic, skinny_gemm_scaled
+    from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    from oracle import skinny_gemm as og
+    g = torch.Generator().manual_seed(11)
+    m, hidden, n = 8, 4096, 1024
+    x = torch.randn(m, hidden, generator=g).to(torch.bfloat16)
+    x[3] *= 40.0
+    r = torch.randn(m, hidden, generator=g).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16)
+    wt = torch.randn(n, hidden, generator=g) * 0.02
+    sw = amax_scale(wt, dim=1)
+    w8 = fp8_quantize(wt, sw)[0]
+    q, _, scales = residual_rms_dynamic(x.cuda(), r.cuda(), w.cuda(), 1e-5)
+    out = skinny_gemm_scaled(q, w8.cuda().t(), scales, sw.reshape(-1).cuda())
+    ref = og.reference_skinny_gemm(q.cpu(), w8.t(), scales.cpu(), sw.reshape(-1), out_dtype=torch.bfloat16)
+    assert torch.allclose(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_dynamic_ops_reject_rows_they_cannot_hold():
+    from hf_rocm_kernels import _capi
+    lib = _capi.load()
+    x = torch.zeros(2, 40000, dtype=torch.bfloat16).cuda()
+    q = torch.zeros(2, 40000, dtype=torch.uint8).cuda()
+    s = torch.zeros(2).cuda()
+    w = torch.zeros(40000, dtype=torch.bfloat16).cuda()
+    rms = lambda cols: lib.hfrk_residual_rms_dynamic(x.data_ptr(), x.data_ptr(), w.data_ptr(), 1e-5, q.data_ptr(), s.data_ptr(),
+                                                     None, 2, cols, 0, _capi.BF16, None)
+    assert rms(36) == _capi.BAD_SHAPE          # cols % 8 != 0
+    assert rms(40000) == _capi.BAD_SHAPE       # wider than the register cache
+    assert lib.hfrk_swiglu_dynamic(x.data_ptr(), q.data_ptr(), s.data_ptr(), None, 1, 20004, 0, _capi.BF16, None) == _capi.BAD_SHAPE
+    assert lib.hfrk_swiglu_dynamic(x.data_ptr() + 2, q.data_ptr(), s.data_ptr(), None, 1, 64, 0, _capi.BF16, None) == _capi.BAD_ALIGNMENT
