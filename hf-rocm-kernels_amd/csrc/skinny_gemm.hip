@@ -1,4 +1,7 @@
-// FP8 (OCP e4m3fn) skinny GEMM for MI355X / gfx950:  D[m,n] (+)= sa[m] * sb[n] * sum_k A[m,k] * W[n,k],  m <= 64.
+// FP8 (OCP e4m3fn) skinny GEMM for MI355X / gfx950:  D[m,n] = base[m,n] + sa[m] * sb[n] * sum_k A[m,k] * W[n,k],  m <= 64.
+//
+// This file holds the host side of the GEMM (workspace, planner, validation, the extern "C" entry points) and the
+// workgroup-cooperative kernel the planner uses above 16 rows; the kernel for m <= 16 is in skinny_gemm_stream.hip.
 //
 // Replaces the reference's persistent producer/consumer kernel and its consumers
 // (csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79, producers/n_full_tiles.cu:4-127,
@@ -613,12 +616,10 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.k = k;
     args.b_stride = b_stride;
     args.d_dtype = d_dtype;
-    args.accumulate = base != nullptr;
     args.panels = p.panels;
     args.slabs = p.slabs;
     args.units = p.panels * p.slabs;
     args.grid = p.grid;
-    args.nbuf = 2;
     args.chunks_q = args.units / p.grid;
     args.chunks_r = args.units % p.grid;
     args.ws = st->ws;

@@ -23,8 +23,8 @@ struct GemmArgs {
     const float* scale_b;
     int sa_stride, sb_stride;
     int m, n, k, b_stride;
-    int d_dtype, accumulate;
-    int panels, slabs, units, grid, nbuf;
+    int d_dtype;             // dtype of D; with the SwiGLU epilogue the 16-bit dtype the projections are rounded to
+    int panels, slabs, units, grid;  // units = panels * slabs
     int chunks_q, chunks_r;  // stream kernel: (panels * slabs) / grid and % grid
     float* ws;
     int* counters;
