@@ -364,3 +364,34 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
         f = out.cpu().float()
         assert not f.isnan().any(), grid
         assert ((f - ref.float()).abs() <= tol).all(), grid
+
+
+def test_benchmarking_helpers_and_the_library_gemm_agree_with_scaled_mm():
+    """The reference times its kernel against torch._scaled_mm (hipBLASLt) and uses it as its oracle
+    (operators/skinny_gemm/reference.py:18-25): same cross-check here, plus the timing helpers on a tiny budget."""
+    from hf_rocm_kernels import skinny_gemm
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    from hf_rocm_kernels.operators.skinny_gemm.benchmarking_fn import benchmark_skinny_gemm
+    from hf_rocm_kernels.operators.swiglu.benchmarking_fn import benchmark_swiglu
+    from hf_rocm_kernels.utils.benchmarking import Bench, benchmark_cuda_graph_no_cache
+    a, b, sa, sw = generate_llama_gemm_data(8, 1024, 2048, seed=12)
+    ours = skinny_gemm(a, b, (sa * sw).contiguous())
+    try:
+        theirs = torch._scaled_mm(a, b, scale_a=sa.reshape(1), scale_b=sw.reshape(1), out_dtype=torch.bfloat16)
+    except Exception as e:  # not every torch build has the fp8 hipBLASLt path
+        theirs = None
+        print("torch._scaled_mm unavailable:", e)
+    if theirs is not None:
+        assert torch.allclose(ours.float(), theirs.float(), rtol=1e-2, atol=1e-2)
+    mean, std = benchmark_skinny_gemm(8, 1024, 2048, {}, graph_size=2, warmups=1, iterations=4)
+    assert 0 < mean < 1e4 and std >= 0
+    med, _ = benchmark_skinny_gemm(8, 1024, 2048, dict(split_k=4, A_producers=2, B_producers=6, consumers=2, a_lanes=2,
+                                                        b_lanes=3, qsize=4, op_m=16, ops=8),
+                                   graph_size=2, warmups=1, iterations=4, mode="median")
+    assert 0 < med < 1e4
+    assert 0 < benchmark_swiglu(4, 1024, -1, graph_size=2, warmups=1, iterations=4) < 1e4
+    t = benchmark_cuda_graph_no_cache(lambda x: x.add_(1), (torch.zeros(1024, device="cuda"),), {}, graph_size=2, warmups=1, iterations=4)
+    assert 0 < t < 1e4
+    bench = Bench()
+    bench.add_measure("add", 1024, lambda: torch.zeros(1024, device="cuda").add_(1), rep=4)
+    assert bench.table("n")["add"][0] > 0

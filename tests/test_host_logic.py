@@ -251,3 +251,49 @@ def test_data_generators_are_seeded_and_follow_the_recipes():
     assert x.dtype == torch.bfloat16 and sc is not None and nb.shape == (3, 16) and 1e-5 <= eps < 2e-5
     gu, sc, nb = generate_swiglu_data(3, 32, 0, seed=3, device="cpu")
     assert gu.shape == (3, 64) and nb is None
+
+
+def test_package_reference_functions_agree_with_the_oracle():
+    """The torch references the package exports for its users (as the reference package does) are a second,
+    independently written statement of the same arithmetic as the oracle: bit-equal on the CPU."""
+    from hf_rocm_kernels.operators.residual_rms import precise_residual_rms, reference_residual_rms
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data, reference_skinny_gemm
+    from hf_rocm_kernels.operators.swiglu import reference_swiglu
+    from oracle import residual_rms as orms
+    from oracle import skinny_gemm as og
+    from oracle import swiglu as osw
+    a, b, sa, sw = generate_llama_gemm_data(5, 96, 512, seed=2, device="cpu", per_token=True, per_channel=True)
+    base = torch.randn(5, 96, generator=torch.Generator().manual_seed(1)).to(torch.float16)
+    assert torch.equal(reference_skinny_gemm(a, b, sa, sw), og.reference_skinny_gemm(a, b, sa, sw))
+    assert torch.equal(reference_skinny_gemm(a, b, sa, sw, output=base), og.reference_skinny_gemm(a, b, sa, sw, output=base))
+    g = torch.Generator().manual_seed(4)
+    for dtype in (torch.float16, torch.bfloat16):
+        x, r = torch.randn(3, 64, generator=g).to(dtype), torch.randn(3, 64, generator=g).to(dtype)
+        w = torch.randn(64, generator=g).to(dtype)
+        scale = torch.tensor([1.7])
+        for s in (scale, None):
+            mine, ref = reference_residual_rms(x, r, w, 1e-5, s), orms.reference_residual_rms(x, r, w, 1e-5, s)
+            assert torch.equal(mine[0].float(), ref[0].float()) and torch.equal(mine[1], ref[1])
+            pm, pr = precise_residual_rms(x, r, w, 1e-5, s), orms.precise_residual_rms(x, r, w, 1e-5, s)
+            # float64 with the factors multiplied in another order: equal to the last bits, and equal once quantised
+            assert torch.allclose(pm[0].double(), pr[0].double(), rtol=1e-14, atol=0) and torch.equal(pm[1], pr[1])
+            assert s is None or torch.equal(pm[0].float(), pr[0].float())
+        gu = torch.randn(3, 128, generator=g).mul(3).to(dtype)
+        assert torch.equal(reference_swiglu(gu, scale).float(), osw.reference_swiglu(gu, scale).float())
+
+
+def test_bench_table_bookkeeping():
+    from hf_rocm_kernels.utils.benchmarking import Bench, randomize_tensors
+    b = Bench.__new__(Bench)  # the constructor queries the GPU
+    b._measures = {}
+    b.add_raw_measure("torch", 8, 10.0)
+    b.add_raw_measure("ours", 8, 4.0)
+    b.add_raw_measure("ours", 16, 5.0)
+    b.add_speedup_column("torch", "ours")
+    t = b.table("M")
+    assert t["M"] == [8, 16] and t["Speedup"] == [2.5, "-"] and t["torch"] == [10.0, "-"]
+    with pytest.raises(ValueError):
+        b.add_speedup_column("missing", "ours")
+    x = torch.zeros(4, 4, dtype=torch.float16)
+    y = randomize_tensors(x)
+    assert y.shape == x.shape and y.dtype == x.dtype and not torch.equal(x, y) and randomize_tensors(3) == 3
