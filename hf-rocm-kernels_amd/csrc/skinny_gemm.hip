@@ -463,16 +463,52 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     return fill_stream_plan(m, n, k, row_tiles, false, 0, plan);
 }
 
+// 17 <= m <= 64 (valid from 1): the waves of a workgroup split K windows of 8*wave_k bytes, activations in registers
+// (skinny_gemm_ksplit.hip).  wave_k 512 keeps twice the bytes in flight and halves the window count, 256 makes
+// twice the units: take the one whose busiest workgroup streams fewer bytes.
+static int fill_ksplit_plan(int m, int n, int k, int wave_k, int grid_hint, hfrk_gemm_plan* plan) {
+    const int mt = (m + 15) / 16;
+    if (!ksplit_variant_exists(mt, wave_k)) return HFRK_INVALID_CONFIG;
+    if (k % (8 * wave_k) != 0) return HFRK_INVALID_CONFIG;
+    const long tiles = (n + 15) / 16, windows = k / (8 * wave_k);
+    const long units = tiles * windows;
+    if (tiles * mt > kMaxPanels) return HFRK_BAD_SHAPE;                          // one arrival counter per 16x16 tile
+    if (windows > 1 && (size_t)units * mt * 256 > kWsFloats) return HFRK_BAD_SHAPE;  // a 16x16 fp32 share per unit and tile
+    long grid = grid_hint > 0 ? grid_hint : kNumCU;
+    if (grid > units) grid = units;
+    if (grid >= 8) grid -= grid % 8;
+    plan->m_tiles = mt;
+    plan->wn = -1;
+    plan->wk = wave_k / 256;
+    plan->ch = 0;
+    plan->grid = (int)grid;
+    plan->panels = (int)tiles;
+    plan->slabs = (int)windows;
+    plan->lds_bytes = ksplit_lds_bytes(mt, wave_k);
+    return HFRK_SUCCESS;
+}
+
+// The planner uses this decomposition only when one window of 256 or 512 bytes per wave covers K (k = 2048 or 4096):
+// then a unit is finished inside its workgroup.  With several windows every unit makes a workspace round trip
+// (store, acknowledge, counter) on the critical path of its workgroup, and with 1 KB per wave (k = 8192, up to 32
+// rows) the kernel sits at 254 registers; measured, the workgroup kernel is faster in both cases.
+static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (k != 2048 && k != 4096) return HFRK_INVALID_CONFIG;
+    return fill_ksplit_plan(m, n, k, k / 8, 0, plan);
+}
+
 // Which decomposition for which shape.  The rules are measurements on MI355X over the Llama-3 8B/70B linears
 // (sweeps of every decomposition at m = 1..64), not a model:
 //   m <= 16          wave-stream kernel (activations per wave from L2: cheap up to 16 rows)
-//   m  > 16          workgroup kernel, which stages the activation slab once per workgroup in LDS:
+//   m  > 16          K-split kernel (activations in registers) when one window of it covers k; otherwise the
+//                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
 //                    4 row waves x 2 K waves almost everywhere; 2 x 4 for small weights (more K parallelism where a
 //                    workgroup only gets a few units); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (m <= 16) return make_stream_plan(m, n, k, plan);
+    if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     const int mt = (m + 15) / 16;
     const double weight_mb = (double)n * k / 1.0e6;
     int first = 4;
@@ -506,6 +542,17 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 
 static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p) {
     if (swiglu && p->wn != 0) return HFRK_INVALID_CONFIG;  // the fused epilogue exists in the wave-stream kernel only
+    if (p->wn == -1) {  // K-split decomposition: wk = wave_k / 256
+        hfrk_gemm_plan want;
+        const int rc = fill_ksplit_plan(m, n, k, p->wk * 256, p->grid, &want);
+        if (rc != HFRK_SUCCESS) return rc;
+        if (p->grid < 1 || p->grid > kNumCU || p->grid > (long)want.panels * want.slabs) return HFRK_INVALID_CONFIG;
+        if (p->m_tiles != want.m_tiles || p->ch != 0 || p->panels != want.panels || p->slabs != want.slabs ||
+            p->lds_bytes != want.lds_bytes)
+            return HFRK_INVALID_CONFIG;
+        if ((long)want.panels * want.slabs * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;
+        return HFRK_SUCCESS;
+    }
     if (p->wn == 0) {  // wave-stream decomposition: wk = row tiles per chunk, ch = activation loads
         if (m > kStreamMaxM || !stream_variant_exists(p->ch, p->wk, swiglu) || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
         if (p->m_tiles != (p->ch + 3) / 4) return HFRK_INVALID_CONFIG;
@@ -625,6 +672,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.ws = st->ws;
     args.counters = st->counters;
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
+    if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, p.lds_bytes, stream);
     switch (p.m_tiles) {
         case 1: return launch_mt<1>(args, p, stream);
         case 2: return launch_mt<2>(args, p, stream);

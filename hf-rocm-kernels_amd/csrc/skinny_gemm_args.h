@@ -45,4 +45,14 @@ constexpr bool stream_variant_exists(int act_loads, int row_tiles, bool swiglu =
                   : (row_tiles == 1 && act_loads >= 1 && act_loads <= 4) || (row_tiles == 2 && act_loads >= 3 && act_loads <= 8);
 }
 
+// K-split kernel (skinny_gemm_ksplit.hip): the 8 waves of a workgroup split a K window of 8*wave_k bytes
+// (wave_k = 256, 512, or 1024 with m_tiles <= 2), activations in registers.  Needs k % (8*wave_k) == 0.
+int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, int lds_bytes, hipStream_t stream);
+constexpr bool ksplit_variant_exists(int m_tiles, int wave_k) {
+    return m_tiles >= 1 && (((wave_k == 256 || wave_k == 512) && m_tiles <= 4) || (wave_k == 1024 && m_tiles <= 2));
+}
+constexpr int ksplit_lds_bytes(int m_tiles, int wave_k) {
+    return kGemmWaves * (wave_k / 256) * kTileBytes + 2 * kGemmWaves * m_tiles * 1024;
+}
+
 }  // namespace hfrk

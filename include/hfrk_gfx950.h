@@ -50,16 +50,20 @@ enum hfrk_epilogue { HFRK_EPILOGUE_NONE = 0, HFRK_EPILOGUE_SWIGLU = 1 };
  * hfrk_skinny_gemm_ex() by an autotuner (counterpart of the knob table in
  * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102 and benchmarks/skinny_gemm/grid_search.py). */
 typedef struct hfrk_gemm_plan {
-    int m_tiles;   /* ceil(m/16): 16-row activation tiles (wave-stream: 1..2, workgroup: 1..4) */
-    int wn;        /* 0: wave-stream decomposition (m <= 32), every wave streams its own run of chunks.
-                      1,2,4,8: workgroup decomposition, wn waves spread over output rows (16 weight rows each) */
-    int wk;        /* workgroup decomposition: waves spread over K, wn*wk = 8.
-                      wave-stream: 16-row weight tiles per chunk, 1 (m <= 16) or 2 (9 <= m <= 32) */
-    int ch;        /* workgroup decomposition: 256-byte K chunks each wave streams per slab (1 or 2).
-                      wave-stream: 16-byte activation loads per lane and chunk, ceil(m/4) */
+    int m_tiles;   /* ceil(m/16): 16-row activation tiles (wave-stream: 1..2, others: 1..4) */
+    int wn;        /* which decomposition:
+                       0          wave-stream (m <= 32): every wave streams its own run of chunks
+                      -1          K-split (k % (2048*wk) == 0): the 8 waves of a workgroup split K, activations in registers
+                       1,2,4,8    workgroup: wn waves spread over output rows (16 weight rows each), wk over K */
+    int wk;        /* workgroup: waves spread over K, wn*wk = 8.  wave-stream: 16-row weight tiles per chunk (1 or 2).
+                      K-split: bytes of K per wave / 256 (1, 2, or 4 with m_tiles <= 2) */
+    int ch;        /* workgroup: 256-byte K chunks each wave streams per slab (1 or 2).
+                      wave-stream: 16-byte activation loads per lane and chunk, ceil(m/4).  K-split: 0 */
     int grid;      /* persistent workgroups launched */
-    int panels;    /* workgroup decomposition: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n / (16*wk)) row groups */
-    int slabs;     /* workgroup decomposition: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per group */
+    int panels;    /* workgroup: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n / (16*wk)) row groups.
+                      K-split: ceil(n/16) row tiles */
+    int slabs;     /* workgroup: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per group.
+                      K-split: k / (2048*wk) windows */
     int lds_bytes; /* dynamic LDS per workgroup */
 } hfrk_gemm_plan;
 

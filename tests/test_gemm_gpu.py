@@ -65,6 +65,11 @@ def all_plans(m, n, k):
             groups = (n + 16 * rt - 1) // (16 * rt)
             for grid in sorted({min(g, groups * kc) for g in (256, 200, 7, 512, 1)}):
                 plans.append(_capi.GemmPlan((ma + 3) // 4, 0, rt, ma, grid, groups, kc, 8 * (rt + (ma + 3) // 4) * 4096))
+    for wave_k in (256, 512, 1024):  # K-split decomposition
+        if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
+            tiles, windows = (n + 15) // 16, k // (8 * wave_k)
+            for grid in sorted({min(g, tiles * windows) for g in (256, 200, 7, 1)}):
+                plans.append(_capi.GemmPlan(mt, -1, wave_k // 256, 0, grid, tiles, windows, 8 * (wave_k // 256) * 4096 + 16 * mt * 1024))
     for wn in (1, 2, 4, 8):
         wk = 8 // wn
         for ch in (1, 2):
@@ -95,7 +100,8 @@ def test_default_plan_matches_oracle(m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
                                    (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024),
-                                   (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096)])
+                                   (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096),
+                                   (32, 1040, 8192), (48, 4096, 4096), (9, 528, 16384)])
 def test_every_plan_gives_the_same_answer(m, n, k):
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=7)

@@ -129,6 +129,16 @@ def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
             assert who == list(range(_stream_owner(plan, lo), _stream_owner(plan, hi - 1) + 1)), (t, who)
         return
     assert m > 16
+    if plan.wn == -1:  # K-split decomposition: units = (window, row tile), window-major, split like the stream chunks
+        wave_k = 256 * plan.wk
+        assert wave_k in (256, 512) and k == 8 * wave_k and plan.ch == 0 and plan.m_tiles == (m + 15) // 16
+        assert plan.panels == -(-n // 16) and plan.slabs == k // (8 * wave_k)
+        assert 1 <= plan.grid <= min(256, plan.panels * plan.slabs)
+        assert plan.lds_bytes == 8 * plan.wk * 4096 + 16 * plan.m_tiles * 1024 <= 160 * 1024
+        ranges = _stream_ranges(plan)
+        assert ranges[0][0] == 0 and ranges[-1][1] == plan.panels * plan.slabs
+        assert all(a[1] == b[0] and a[0] < a[1] for a, b in zip(ranges, ranges[1:]))
+        return
     assert plan.m_tiles == (m + 15) // 16 and plan.wn * plan.wk == 8 and plan.ch in (1, 2)
     ks = 256 * plan.wk * plan.ch
     assert k % ks == 0 and plan.slabs == k // ks and plan.panels == -(-n // (16 * plan.wn))
