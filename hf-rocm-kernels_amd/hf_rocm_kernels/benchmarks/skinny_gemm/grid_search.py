@@ -1,0 +1,139 @@
+"""Time every decomposition the library offers for a GEMM shape and report the fastest next to the planner's choice.
+
+Counterpart of the reference package's benchmarks/skinny_gemm/grid_search.py, which walks its knob tuples
+(a_lanes, b_lanes, qsize, op_m, ops).  Here the search space is `hfrk_gemm_plan`: the wave-stream, K-split and
+workgroup decompositions with their parameters and a few grid sizes, passed to `hfrk_skinny_gemm_ex`.  The rules in
+the library's planner were read off sweeps like this one.  Usage, from the repository root:
+    python hf-rocm-kernels_amd/hf_rocm_kernels/benchmarks/skinny_gemm/grid_search.py -m 8 32 -n 4096 -k 4096 [--json out.json]
+"""
+import argparse
+import ctypes
+import itertools
+import json
+import os
+import sys
+from typing import Dict, List
+
+if __package__ in (None, ""):
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", ".."))
+
+import torch  # noqa: E402
+
+from hf_rocm_kernels import _capi  # noqa: E402
+
+
+def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.GemmPlan]:
+    """Every plan `hfrk_skinny_gemm_ex` accepts for the shape, over the given grid sizes."""
+    mt = (m + 15) // 16
+    plans = []
+    if m <= 32:  # wave-stream: row tiles per chunk 1 or 2
+        ma, kc = (m + 3) // 4, k // 256
+        for rt in (1, 2):
+            if (rt == 1 and ma <= 4) or (rt == 2 and 3 <= ma <= 8):
+                groups = -(-n // (16 * rt))
+                for g in grids:
+                    plans.append(_capi.GemmPlan((ma + 3) // 4, 0, rt, ma, min(g, groups * kc), groups, kc,
+                                                8 * (rt + (ma + 3) // 4) * 4096))
+    for wave_k in (256, 512, 1024):  # K-split
+        if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
+            tiles, windows = -(-n // 16), k // (8 * wave_k)
+            if windows > 1 and tiles * windows * mt * 256 > 2 * 1024 * 8 * 4 * 256:
+                continue  # more shares than the workspace holds
+            for g in grids:
+                plans.append(_capi.GemmPlan(mt, -1, wave_k // 256, 0, min(g, 256, tiles * windows), tiles, windows,
+                                            8 * (wave_k // 256) * 4096 + 16 * mt * 1024))
+    for wn, ch in itertools.product((1, 2, 4, 8), (1, 2)):  # workgroup
+        wk = 8 // wn
+        ks = 256 * wk * ch
+        lds = 8 * 4096 + 2 * 16 * mt * ks + 16
+        if k % ks or lds > 160 * 1024:
+            continue
+        panels, slabs = -(-n // (16 * wn)), k // ks
+        for g in grids:
+            plans.append(_capi.GemmPlan(mt, wn, wk, ch, min(g, panels * slabs), panels, slabs, lds))
+    return plans
+
+
+def describe(p: _capi.GemmPlan) -> str:
+    if p.wn == 0:
+        return f"wave-stream row_tiles={p.wk} act_loads={p.ch} grid={p.grid}"
+    if p.wn == -1:
+        return f"k-split wave_k={256 * p.wk} windows={p.slabs} grid={p.grid}"
+    return f"workgroup wn={p.wn} wk={p.wk} ch={p.ch} grid={p.grid}"
+
+
+def time_plan(lib, arena: torch.Tensor, m: int, n: int, k: int, plan, reps: int) -> float:
+    """Median microseconds per call from a graph over as many distinct weights as fit the arena (HBM-cold)."""
+    nbuf = max(2, min(64, arena.numel() // (n * k)))
+    a = arena[: m * k]
+    scale = torch.ones(1, device=arena.device)
+    out = torch.zeros((m, n), dtype=torch.bfloat16, device=arena.device)
+    weights = [arena[i * n * k:(i + 1) * n * k] for i in range(nbuf)]
+    ref = None if plan is None else ctypes.byref(plan)
+
+    def call(w: torch.Tensor, stream: int) -> None:
+        status = lib.hfrk_skinny_gemm_ex(a.data_ptr(), w.data_ptr(), out.data_ptr(), scale.data_ptr(), 0, None, 0, m, n, k, k,
+                                         _capi.BF16, 0, ref, stream)
+        if status != 0:
+            raise RuntimeError(f"plan rejected with status {status}: {_capi.status_string(status)}")
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        call(weights[0], side.cuda_stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for w in weights:
+            call(w, torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    samples = []
+    for _ in range(reps):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        end.record()
+        end.synchronize()
+        samples.append(start.elapsed_time(end) * 1e3 / nbuf)
+    samples.sort()
+    return samples[len(samples) // 2]
+
+
+def main() -> None:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--m", "-m", type=int, nargs="+", default=[8])
+    parser.add_argument("--n", "-n", type=int, nargs="+", default=[4096])
+    parser.add_argument("--k", "-k", type=int, nargs="+", default=[4096])
+    parser.add_argument("--grids", type=int, nargs="+", default=[256])
+    parser.add_argument("--reps", type=int, default=20)
+    parser.add_argument("--top", type=int, default=3)
+    parser.add_argument("--json", default=None, help="write the full table here")
+    args = parser.parse_args()
+    lib = _capi.load()
+    _capi.check(lib.hfrk_init(), "hfrk_init")
+    arena = torch.randint(0, 120, (1 << 30,), dtype=torch.uint8, device="cuda")  # finite fp8 codes
+    table: Dict[str, dict] = {}
+    for m, n, k in itertools.product(args.m, args.n, args.k):
+        chosen = _capi.plan(m, n, k)
+        t_default = time_plan(lib, arena, m, n, k, None, args.reps)
+        rows = []
+        for p in candidate_plans(m, n, k, args.grids):
+            try:
+                rows.append((time_plan(lib, arena, m, n, k, p, args.reps), describe(p), p.as_dict()))
+            except RuntimeError as e:
+                print(f"# {describe(p)}: {e}")
+        rows.sort(key=lambda r: r[0])
+        gbps = (n * k + m * k + 2 * m * n) / t_default / 1e3
+        print(f"m={m} n={n} k={k}: planner -> {describe(chosen)}: {t_default:.2f} us ({gbps:.0f} GB/s)")
+        for t, text, _ in rows[: args.top]:
+            print(f"    {t:8.2f} us  {text}")
+        table[f"{m}x{n}x{k}"] = {"planner": chosen.as_dict(), "planner_us": t_default,
+                                 "plans": [{"us": t, "plan": d} for t, _, d in rows]}
+    if args.json:
+        with open(args.json, "w") as f:
+            json.dump(table, f, indent=1)
+
+
+if __name__ == "__main__":
+    main()
