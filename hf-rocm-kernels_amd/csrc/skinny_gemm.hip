@@ -37,7 +37,9 @@ namespace hfrk {
 // 32-bit on purpose (64-bit division is a long instruction sequence); the host checks units * (grid + 1) < 2^31.
 __device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (int)(((uint32_t)g * (uint32_t)units) / (uint32_t)grid); }
 
-template <int MT, int WN, int WK, int CH>
+// PACKED: the weight is in the pre-packed layout (pack_weight.hip), chunk (tile, kc) at (tile * k/256 + kc) * 4096 in
+// MFMA operand order: the loads are 1 KB contiguous per instruction and the chunk skips the transposition tile.
+template <int MT, int WN, int WK, int CH, bool PACKED>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArgs a) {
     static_assert(WN * WK == kGemmWaves, "a workgroup is 8 waves");
     constexpr int KS = 256 * WK * CH;        // bytes of K per slab
@@ -64,7 +66,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     const int u0 = unit_begin(g, U, G), u1 = unit_begin(g + 1, U, G);
     if (u0 >= u1) return;  // cannot happen when grid <= units; uniform for the whole workgroup
 
-    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, PACKED ? (uint32_t)((a.n + 15) >> 4) * (uint32_t)a.k * 16u
+                                                                : (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     uint16_t* const D = reinterpret_cast<uint16_t*>(a.D);
     const uint16_t* const Dbase = reinterpret_cast<const uint16_t*>(a.base);  // added to the product when not null
@@ -128,13 +131,22 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // Weight chunk c of unit (ip, is) into register set X.
     auto issue_chunk = [&](auto sel, int c, bool in_range) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
-        const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
-                                             (uint32_t)(c * WK + wk) * 256u
-                                       : 0x80000000u;
+        if constexpr (PACKED) {
+            // a tile past the last one (n not a multiple of 16*WN) lies beyond the buffer and reads as zero
+            const uint32_t chunk = (uint32_t)(ip * WN + wn) * ((uint32_t)a.k >> 8) + (uint32_t)phys_slab(ip, is) * (WK * CH) + (uint32_t)(c * WK + wk);
+            const uint32_t base = in_range ? chunk * (uint32_t)kTileBytes + (uint32_t)lane * 16u : 0x80000000u;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(
-                w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+            for (int t = 0; t < 4; ++t)
+                wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(base + (uint32_t)t * 1024u), 0, 2 /* nt */);
+        } else {
+            const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
+                                                 (uint32_t)(c * WK + wk) * 256u
+                                           : 0x80000000u;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(
+                    w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+        }
     };
     // Epilogue inputs of unit (ip, is) if it opens a panel, then move on to the next unit.
     auto issue_done = [&](bool in_range) __attribute__((always_inline)) {
@@ -207,8 +219,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         const uint8_t* const act = act_all + buf * ACT_BYTES;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
+            v4i wcur[4];  // PACKED: the chunk's operands, out of the way of the next request
 #pragma unroll
-            for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tb + wr_off[t]) = wq[X][c][t];
+            for (int t = 0; t < 4; ++t) {
+                if constexpr (PACKED) wcur[t] = wq[X][c][t];
+                else *reinterpret_cast<v4i*>(tb + wr_off[t]) = wq[X][c][t];
+            }
             issue_chunk(sel, c, next_in_range);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -216,8 +232,14 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             const int kblk = c * WK + wk;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const v4i wlo = *reinterpret_cast<const v4i*>(tb + li * 256 + rd_off[h]);
-                const v4i whi = *reinterpret_cast<const v4i*>(tb + li * 256 + (rd_off[h] ^ 16));
+                v4i wlo, whi;
+                if constexpr (PACKED) {
+                    wlo = wcur[2 * h];
+                    whi = wcur[2 * h + 1];
+                } else {
+                    wlo = *reinterpret_cast<const v4i*>(tb + li * 256 + rd_off[h]);
+                    whi = *reinterpret_cast<const v4i*>(tb + li * 256 + (rd_off[h] ^ 16));
+                }
                 const v8i wop = {wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
@@ -577,9 +599,9 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p)
     return HFRK_SUCCESS;
 }
 
-template <int MT, int WN, int WK, int CH>
-static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_kernel<MT, WN, WK, CH>;
+template <int MT, int WN, int WK, int CH, bool PACKED>
+static int launch_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    auto kern = skinny_gemm_kernel<MT, WN, WK, CH, PACKED>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -590,6 +612,12 @@ static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);
     HFRK_HIP_TRY(hipGetLastError());
     return HFRK_SUCCESS;
+}
+
+template <int MT, int WN, int WK, int CH>
+static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    return args.packed ? launch_packing<MT, WN, WK, CH, true>(args, lds_bytes, stream)
+                       : launch_packing<MT, WN, WK, CH, false>(args, lds_bytes, stream);
 }
 
 template <int MT>
@@ -608,7 +636,8 @@ static int launch_mt(const GemmArgs& args, const hfrk_gemm_plan& p, hipStream_t 
 // D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
 static int gemm_launch(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
                        const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k, int b_stride,
-                       int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream) {
+                       int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream, bool packed = false) {
+    if (packed) b_stride = k;
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (d_dtype != HFRK_F16 && d_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
@@ -662,6 +691,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.n = n;
     args.k = k;
     args.b_stride = b_stride;
+    args.packed = packed ? 1 : 0;
     args.d_dtype = d_dtype;
     args.panels = p.panels;
     args.slabs = p.slabs;
@@ -739,6 +769,13 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
                            int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
     return hfrk::gemm_launch(A, B, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, m, n, k, b_stride, d_dtype,
                              epilogue, plan, static_cast<hipStream_t>(stream));
+}
+
+int hfrk_skinny_gemm_packed(const void* A, const void* B_packed, void* D, const void* base, const float* scale_a,
+                            int sa_stride, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
+                            int k, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
+    return hfrk::gemm_launch(A, B_packed, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, m, n, k, k, d_dtype,
+                             epilogue, plan, static_cast<hipStream_t>(stream), true);
 }
 
 }  // extern "C"

@@ -23,6 +23,7 @@ struct GemmArgs {
     const float* scale_b;
     int sa_stride, sb_stride;
     int m, n, k, b_stride;
+    int packed;              // B is in the pre-packed layout of pack_weight.hip (b_stride unused)
     int d_dtype;             // dtype of D; with the SwiGLU epilogue the 16-bit dtype the projections are rounded to
     int panels, slabs, units, grid;  // units = panels * slabs
     int chunks_q, chunks_r;  // stream kernel: (panels * slabs) / grid and % grid

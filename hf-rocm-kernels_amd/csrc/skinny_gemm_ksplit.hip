@@ -23,7 +23,10 @@
 
 namespace hfrk {
 
-template <int MT, int KW>
+// PACKED: the weight is in the pre-packed layout (pack_weight.hip), chunk (tile, kc) at (tile * k/256 + kc) * 4096 in
+// MFMA operand order: a wave's piece of a unit is KW/256 contiguous chunks, the loaded registers are the operands,
+// and each chunk of the next unit is requested as soon as the MFMAs of the current one have taken its registers.
+template <int MT, int KW, bool PACKED>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const GemmArgs a) {
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kCoherent = 17;     // sc0 | sc1
@@ -52,7 +55,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     int win = (int)(u0 / (uint32_t)T);
     int tile = (int)(u0 - (uint32_t)win * (uint32_t)T);
 
-    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, PACKED ? (uint32_t)T * (uint32_t)a.k * 16u
+                                                                : (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
     const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
@@ -66,13 +70,23 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)wv * KW + (uint32_t)li * 16u;
     v4i wq[KCH][4];
     int itile = tile, iwin = win;  // unit being requested
-    auto issue_unit = [&]() __attribute__((always_inline)) {
-        const uint32_t base = (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)iwin * (8u * KW);
+    // column chunk c of the wave's piece of unit (itile, iwin); `base` is the unit's row-major offset
+    auto issue_chunk = [&](int c, uint32_t base) __attribute__((always_inline)) {
+        if constexpr (PACKED) {
+            const uint32_t chunk = (uint32_t)itile * ((uint32_t)a.k >> 8) + ((uint32_t)iwin * 8u + (uint32_t)wv) * KCH + (uint32_t)c;
 #pragma unroll
-        for (int c = 0; c < KCH; ++c)
+            for (int t = 0; t < 4; ++t)
+                wq[c][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(chunk * (uint32_t)kTileBytes + (uint32_t)t * 1024u + (uint32_t)lane * 16u), 0, 2 /* nt */);
+        } else {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
                 wq[c][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride + (uint32_t)c * 256u), 0, 2 /* nt */);
+        }
+    };
+    auto issue_unit = [&]() __attribute__((always_inline)) {
+        const uint32_t base = (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)iwin * (8u * KW);
+#pragma unroll
+        for (int c = 0; c < KCH; ++c) issue_chunk(c, base);
     };
     if (count > 0) issue_unit();
     __builtin_amdgcn_sched_barrier(0);  // the first weight request goes out before anything else is set up
@@ -170,19 +184,23 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     // ---- unit loop ----------------------------------------------------------------------------------------------------
 #pragma unroll 1
     for (int i = 0; i < count; ++i) {
+        if constexpr (!PACKED) {
 #pragma unroll
-        for (int c = 0; c < KCH; ++c)
+            for (int c = 0; c < KCH; ++c)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + c * kTileBytes + wr_off[t]) = wq[c][t];
+                for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + c * kTileBytes + wr_off[t]) = wq[c][t];
+        }
         const bool more = i + 1 < count;
         bool new_window = false;
-        if (more) {  // registers are free again: request the next unit before the LDS reads and MFMAs
+        if (more) {  // row-major: registers are free again, request the next unit before the LDS reads and MFMAs
             if (++itile == T) { itile = 0; ++iwin; new_window = true; }
-            issue_unit();
+            if constexpr (!PACKED) issue_unit();
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if constexpr (!PACKED) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
         v4f acc[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
@@ -190,16 +208,27 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
         for (int c = 0; c < KCH; ++c) {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const v4i lo = *reinterpret_cast<const v4i*>(tw + c * kTileBytes + rd_off[h]);
-                const v4i hi = *reinterpret_cast<const v4i*>(tw + c * kTileBytes + (rd_off[h] ^ 16));
+                v4i lo, hi;
+                if constexpr (PACKED) {
+                    lo = wq[c][2 * h];
+                    hi = wq[c][2 * h + 1];
+                } else {
+                    lo = *reinterpret_cast<const v4i*>(tw + c * kTileBytes + rd_off[h]);
+                    hi = *reinterpret_cast<const v4i*>(tw + c * kTileBytes + (rd_off[h] ^ 16));
+                }
                 const v8i wop = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, areg[mt][2 * c + h], acc[mt], 0, 0, 0, 0, 0, 0);
             }
+            if constexpr (PACKED) {
+                if (more) issue_chunk(c, 0u);
+            }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        if constexpr (!PACKED) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
 
         // sum the eight K pieces: buffer i & 1 (the barrier of the next unit separates its reuse from these reads)
         v4f* const rb = red + (i & 1) * kRedBuf;
@@ -252,9 +281,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     }
 }
 
-template <int MT, int KW>
-static int launch_ksplit_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_ksplit_kernel<MT, KW>;
+template <int MT, int KW, bool PACKED>
+static int launch_ksplit_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    auto kern = skinny_gemm_ksplit_kernel<MT, KW, PACKED>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -265,6 +294,12 @@ static int launch_ksplit_one(const GemmArgs& args, int lds_bytes, hipStream_t st
     hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);
     HFRK_HIP_TRY(hipGetLastError());
     return HFRK_SUCCESS;
+}
+
+template <int MT, int KW>
+static int launch_ksplit_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    return args.packed ? launch_ksplit_packing<MT, KW, true>(args, lds_bytes, stream)
+                       : launch_ksplit_packing<MT, KW, false>(args, lds_bytes, stream);
 }
 
 int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, int lds_bytes, hipStream_t stream) {

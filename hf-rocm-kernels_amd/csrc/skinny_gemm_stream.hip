@@ -38,7 +38,9 @@ namespace hfrk {
 // SWIGLU: the weight is a gate_up projection (gate rows [0, n/2), up rows [n/2, n)); a chunk pairs gate tile t with
 // up tile t (RT = 2) and the epilogue stores fp8(silu(gate) * up / out_scale) into D [m, n/2] instead of the two
 // 16-bit projections -- the SwiGLU kernel of csrc/op_src/swiglu/swiglu_vectorized.cu:27-97 as a GEMM epilogue.
-template <int MA, int RT, bool SWIGLU>
+// PACKED: the weight is in the pre-packed layout (pack_weight.hip): chunk (tile, kc) is 4 KB at
+// (tile * KC + kc) * 4096, already in MFMA operand order, so a chunk is one contiguous read and needs no LDS pass.
+template <int MA, int RT, bool SWIGLU, bool PACKED>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const GemmArgs a) {
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kCoherent = 17;  // sc0 | sc1
@@ -73,7 +75,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     int kc = (int)(w0 - (uint32_t)tile * (uint32_t)KC);
 
     // ---- first request, as early as possible ---------------------------------------------------------------------
-    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, PACKED ? (uint32_t)((a.n + 15) >> 4) * (uint32_t)KC * (uint32_t)kTileBytes
+                                                                : (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
     const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
@@ -86,9 +89,19 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
 #pragma unroll
         for (int t = 0; t < MA; ++t)
             aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+        if constexpr (PACKED) {
+            // 16-row tile of row group t: RT*t + rt, or with SWIGLU t (gate) and n/32 + t (up); a tile past the last
+            // one (odd tile count, RT = 2) is out of the buffer's range and reads as zero
 #pragma unroll
-        for (int t = 0; t < 4 * RT; ++t)
-            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(SWIGLU ? (t / 4) * (a.n >> 1) + 4 * (t % 4) : 4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+            for (int t = 0; t < 4 * RT; ++t) {
+                const uint32_t tl = SWIGLU ? (uint32_t)itile + (uint32_t)(t / 4) * (uint32_t)(a.n >> 5) : (uint32_t)itile * RT + (uint32_t)(t / 4);
+                wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)((tl * (uint32_t)KC + (uint32_t)ikc) * (uint32_t)kTileBytes + (uint32_t)(t % 4) * 1024u + (uint32_t)lane * 16u), 0, 2 /* nt */);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4 * RT; ++t)
+                wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(SWIGLU ? (t / 4) * (a.n >> 1) + 4 * (t % 4) : 4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+        }
     };
     if (count > 0) issue_chunk();
     __builtin_amdgcn_sched_barrier(0);  // keep the set-up below behind the first request
@@ -240,8 +253,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     for (int i = 0; i < count; ++i) {
 #pragma unroll
         for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + (t / 4) * kTileBytes + wr_off[t % 4]) = aq[t];
+        v4i wcur[4 * RT];  // PACKED: the chunk's operands, out of the way of the next request
 #pragma unroll
-        for (int t = 0; t < 4 * RT; ++t) *reinterpret_cast<v4i*>(tw + (t / 4) * kTileBytes + wr_off[t % 4]) = wq[t];
+        for (int t = 0; t < 4 * RT; ++t) {
+            if constexpr (PACKED) wcur[t] = wq[t];
+            else *reinterpret_cast<v4i*>(tw + (t / 4) * kTileBytes + wr_off[t % 4]) = wq[t];
+        }
         pre_cur = pre_next;
         if (i + 1 < count) {  // registers are free again: request the next chunk before the LDS reads and MFMAs
             if (++ikc == KC) { ikc = 0; ++itile; }
@@ -256,8 +273,14 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
             v8i wop[RT], aop[MT];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                const v4i lo = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + rd_off[h]);
-                const v4i hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
+                v4i lo, hi;
+                if constexpr (PACKED) {
+                    lo = wcur[4 * rt + 2 * h];
+                    hi = wcur[4 * rt + 2 * h + 1];
+                } else {
+                    lo = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + rd_off[h]);
+                    hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
+                }
                 wop[rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
 #pragma unroll
@@ -383,9 +406,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     }
 }
 
-template <int MA, int RT, bool SWIGLU>
-static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_stream_kernel<MA, RT, SWIGLU>;
+template <int MA, int RT, bool SWIGLU, bool PACKED>
+static int launch_stream_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    auto kern = skinny_gemm_stream_kernel<MA, RT, SWIGLU, PACKED>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -396,6 +419,12 @@ static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t st
     hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);
     HFRK_HIP_TRY(hipGetLastError());
     return HFRK_SUCCESS;
+}
+
+template <int MA, int RT, bool SWIGLU>
+static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    return args.packed ? launch_stream_packing<MA, RT, SWIGLU, true>(args, lds_bytes, stream)
+                       : launch_stream_packing<MA, RT, SWIGLU, false>(args, lds_bytes, stream);
 }
 
 int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream) {

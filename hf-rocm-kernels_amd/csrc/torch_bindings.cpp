@@ -237,16 +237,25 @@ void swiglu_dynamic(at::Tensor& gate_up, at::Tensor& output, at::Tensor& scales,
 //   epilogue 0: D = (base ? base : 0) + scale_a x scale_b x A.B, base a 16-bit [m,n] tensor (D itself, a residual) or None
 //   epilogue 1: B is a gate_up weight [k, 2*inter]; D fp8 [m, inter] = e4m3fn(silu(gate) * up / out_scale), the two
 //               projections rounded to `intermediate_dtype` (0 = float16, 1 = bfloat16) first
-int64_t skinny_gemm_fused(at::Tensor& A, at::Tensor& B, at::Tensor& D, const std::optional<at::Tensor>& base,
-                          at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
+// Shared by skinny_gemm_fused (B = the [k, n] view of a row-major weight) and skinny_gemm_packed (B = the buffer
+// pack_weight wrote, n given by the caller).
+int64_t gemm_fused_common(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, at::Tensor& D,
+                          const std::optional<at::Tensor>& base, at::Tensor& scale_a,
+                          const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
                           int64_t epilogue, int64_t intermediate_dtype) {
     TORCH_CHECK(A.dim() == 2 && A.is_contiguous(), "A must be a contiguous [m, k] tensor");
-    TORCH_CHECK(B.dim() == 2 && B.size(0) == A.size(1) && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
     check_fp8(A, "A");
     check_fp8(B, "B");
+    if (packed) {
+        TORCH_CHECK(n >= 1 && n < (int64_t(1) << 30) && A.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
+        TORCH_CHECK(B.is_contiguous() && (size_t)B.numel() == hfrk_packed_weight_bytes((int)n, (int)A.size(1)) && B.numel() > 0,
+                    "B must be the packed buffer of a [n, k] weight (pack_weight) with k = A.size(1)");
+    } else {
+        TORCH_CHECK(B.dim() == 2 && B.size(0) == A.size(1) && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
+    }
     check_same_device(A, B, "B");
     check_same_device(A, D, "D");
-    const int64_t m = A.size(0), n = B.size(1);
+    const int64_t m = A.size(0);
     TORCH_CHECK(scale_a.scalar_type() == at::kFloat && scale_a.is_contiguous() && (scale_a.numel() == 1 || scale_a.numel() == m),
                 "scale_a must be float32 with 1 or m elements");
     check_same_device(A, scale_a, "scale_a");
@@ -284,9 +293,63 @@ int64_t skinny_gemm_fused(at::Tensor& A, at::Tensor& B, at::Tensor& D, const std
         }
     }
     DeviceScope scope(A);
+    if (packed)
+        return hfrk_skinny_gemm_packed(A.data_ptr(), B.data_ptr(), D.data_ptr(), base_ptr, scale_a.data_ptr<float>(),
+                                       scale_a.numel() == 1 ? 0 : 1, scale_b_ptr, sb_stride, out_scale_ptr, (int)m, (int)n,
+                                       (int)A.size(1), d_dtype, (int)epilogue, nullptr, current_stream(A));
     return hfrk_skinny_gemm_fused(A.data_ptr(), B.data_ptr(), D.data_ptr(), base_ptr, scale_a.data_ptr<float>(),
                                   scale_a.numel() == 1 ? 0 : 1, scale_b_ptr, sb_stride, out_scale_ptr, (int)m, (int)n, (int)A.size(1), (int)B.stride(1), d_dtype, (int)epilogue,
                                   nullptr, current_stream(A));
+}
+
+int64_t skinny_gemm_fused(at::Tensor& A, at::Tensor& B, at::Tensor& D, const std::optional<at::Tensor>& base,
+                          at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
+                          int64_t epilogue, int64_t intermediate_dtype) {
+    TORCH_CHECK(B.dim() == 2, "B must be [k, n] with unit stride along k");
+    return gemm_fused_common(A, B, false, B.size(1), D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype);
+}
+
+// The same on a weight in the load format of hfrk_pack_weight (no reference counterpart).
+int64_t skinny_gemm_packed(at::Tensor& A, at::Tensor& B_packed, int64_t n, at::Tensor& D, const std::optional<at::Tensor>& base,
+                           at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
+                           int64_t epilogue, int64_t intermediate_dtype) {
+    return gemm_fused_common(A, B_packed, true, n, D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype);
+}
+
+bool is_byte_tensor(const at::Tensor& t) {
+    return t.scalar_type() == at::kByte || t.scalar_type() == at::kFloat8_e4m3fn || t.scalar_type() == at::kFloat8_e4m3fnuz;
+}
+
+// Row-major [n, k] fp8 weight -> packed load format; src_format 1 re-encodes e4m3fnuz values as e4m3fn on the way.
+void pack_weight(at::Tensor& src, at::Tensor& dst, int64_t src_format) {
+    TORCH_CHECK(src.dim() == 2 && src.stride(1) == 1 && is_byte_tensor(src), "src must be a [n, k] one-byte tensor with unit stride along k");
+    TORCH_CHECK(src.size(0) < (int64_t(1) << 30) && src.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
+    const int n = (int)src.size(0), k = (int)src.size(1);
+    TORCH_CHECK(is_byte_tensor(dst) && dst.is_contiguous() && (size_t)dst.numel() == hfrk_packed_weight_bytes(n, k) && dst.numel() > 0,
+                "dst must be a contiguous one-byte tensor of hfrk_packed_weight_bytes(n, k) elements (k % 256 == 0)");
+    check_same_device(src, dst, "dst");
+    DeviceScope scope(src);
+    raise_on(hfrk_pack_weight(src.data_ptr(), (int)src.stride(0), (int)src_format, dst.data_ptr(), n, k, current_stream(src)), "pack_weight");
+}
+
+void unpack_weight(at::Tensor& src, at::Tensor& dst) {
+    TORCH_CHECK(dst.dim() == 2 && dst.stride(1) == 1 && is_byte_tensor(dst), "dst must be a [n, k] one-byte tensor with unit stride along k");
+    TORCH_CHECK(dst.size(0) < (int64_t(1) << 30) && dst.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
+    const int n = (int)dst.size(0), k = (int)dst.size(1);
+    TORCH_CHECK(is_byte_tensor(src) && src.is_contiguous() && (size_t)src.numel() == hfrk_packed_weight_bytes(n, k) && src.numel() > 0,
+                "src must be a contiguous one-byte tensor of hfrk_packed_weight_bytes(n, k) elements (k % 256 == 0)");
+    check_same_device(src, dst, "dst");
+    DeviceScope scope(src);
+    raise_on(hfrk_unpack_weight(src.data_ptr(), dst.data_ptr(), (int)dst.stride(0), n, k, current_stream(src)), "unpack_weight");
+}
+
+// e4m3fnuz bytes -> e4m3fn bytes with the same values (dst may be src).
+void reencode_fnuz(at::Tensor& src, at::Tensor& dst) {
+    TORCH_CHECK(is_byte_tensor(src) && is_byte_tensor(dst) && src.is_contiguous() && dst.is_contiguous() && src.numel() == dst.numel(),
+                "src and dst must be contiguous one-byte tensors of the same size");
+    check_same_device(src, dst, "dst");
+    DeviceScope scope(src);
+    raise_on(hfrk_reencode_fnuz(src.data_ptr(), dst.data_ptr(), (size_t)src.numel(), current_stream(src)), "reencode_fnuz");
 }
 
 }  // namespace
@@ -317,6 +380,18 @@ TORCH_LIBRARY(_HFRK_C, ops) {
         "skinny_gemm_fused(Tensor A, Tensor B, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
         "Tensor? out_scale, int epilogue, int intermediate_dtype) -> int");
     ops.impl("skinny_gemm_fused", c10::kCUDA, &skinny_gemm_fused);
+
+    ops.def(
+        "skinny_gemm_packed(Tensor A, Tensor B_packed, int n, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
+        "Tensor? out_scale, int epilogue, int intermediate_dtype) -> int");
+    ops.impl("skinny_gemm_packed", c10::kCUDA, &skinny_gemm_packed);
+
+    ops.def("pack_weight(Tensor src, Tensor! dst, int src_format) -> ()");
+    ops.impl("pack_weight", c10::kCUDA, &pack_weight);
+    ops.def("unpack_weight(Tensor src, Tensor! dst) -> ()");
+    ops.impl("unpack_weight", c10::kCUDA, &unpack_weight);
+    ops.def("reencode_fnuz(Tensor src, Tensor! dst) -> ()");
+    ops.impl("reencode_fnuz", c10::kCUDA, &reencode_fnuz);
 
     ops.def(
         "residual_rms_dynamic(Tensor input, Tensor! residual, Tensor weight, float epsilon, Tensor! output, "

@@ -32,6 +32,10 @@ FP8_E4M3FN = 2
 EPILOGUE_NONE = 0
 EPILOGUE_SWIGLU = 1
 
+# enum hfrk_weight_format
+WEIGHT_E4M3FN = 0
+WEIGHT_E4M3FNUZ = 1
+
 GEMM_MAX_M = 64
 
 
@@ -57,6 +61,11 @@ SIGNATURES = {
     "hfrk_skinny_gemm": (_i, [_p, _p, _p, _p] + [_i] * 14 + [_p]),
     "hfrk_skinny_gemm_ex": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
+    "hfrk_packed_weight_bytes": (ctypes.c_size_t, [_i, _i]),
+    "hfrk_pack_weight": (_i, [_p, _i, _i, _p, _i, _i, _p]),
+    "hfrk_unpack_weight": (_i, [_p, _p, _i, _i, _i, _p]),
+    "hfrk_reencode_fnuz": (_i, [_p, _p, ctypes.c_size_t, _p]),
+    "hfrk_skinny_gemm_packed": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_residual_rms": (_i, [_p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "hfrk_swiglu": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "hfrk_residual_rms_dynamic": (_i, [_p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _p]),

@@ -36,3 +36,8 @@ def _skinny_gemm_scaled(A: Tensor, B: Tensor, D: Tensor, scale_a: Tensor, scale_
 def _skinny_gemm_fused(A: Tensor, B: Tensor, D: Tensor, base, scale_a: Tensor, scale_b: Tensor, out_scale, epilogue: int,
                        intermediate_dtype: int) -> int:
     return torch.ops._HFRK_C.skinny_gemm_fused(A, B, D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)
+
+
+def _skinny_gemm_packed(A: Tensor, B_packed: Tensor, n: int, D: Tensor, base, scale_a: Tensor, scale_b, out_scale, epilogue: int,
+                        intermediate_dtype: int) -> int:
+    return torch.ops._HFRK_C.skinny_gemm_packed(A, B_packed, n, D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)

@@ -4,7 +4,8 @@ import torch
 from torch import Tensor
 
 from ... import _capi
-from .binding import _skinny_gemm, _skinny_gemm_fused, _skinny_gemm_scaled
+from ...utils.weight_format import PackedWeight
+from .binding import _skinny_gemm, _skinny_gemm_fused, _skinny_gemm_packed, _skinny_gemm_scaled
 
 _OUT_DTYPES = (torch.bfloat16, torch.float16)
 
@@ -71,6 +72,17 @@ def _raise_on_status(status: int, what: str) -> None:
         raise RuntimeError(f"{what} rejected the call with status {status}: {_capi.status_string(status)}")
 
 
+def _fused(skinny_a: Tensor, b, output: Tensor, base: Optional[Tensor], scale_a: Tensor, scale_b: Optional[Tensor],
+           out_scale: Optional[Tensor], epilogue: int, intermediate_dtype: int) -> None:
+    """One launch of the fused GEMM on a row-major view or a PackedWeight; raises on a non-zero status."""
+    if isinstance(b, PackedWeight):
+        status = _skinny_gemm_packed(skinny_a, b.data, b.n, output, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)
+        _raise_on_status(status, "skinny_gemm_packed")
+    else:
+        status = _skinny_gemm_fused(skinny_a, b, output, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)
+        _raise_on_status(status, "skinny_gemm_fused")
+
+
 def skinny_gemm(
     skinny_a: Tensor,
     b: Tensor,
@@ -80,7 +92,8 @@ def skinny_gemm(
     """FP8 skinny GEMM: output += scale * skinny_a @ b, fp32 accumulation, one rounding.
     Args (reference: operators/skinny_gemm/wrapped.py:104-128):
         - skinny_a: a float8_e4m3fn tensor of shape (m, k) in row-major format, m <= 64
-        - b: a float8_e4m3fn tensor of shape (k, n) in col-major format (an nn.Linear weight [n, k], transposed)
+        - b: a float8_e4m3fn tensor of shape (k, n) in col-major format (an nn.Linear weight [n, k], transposed),
+          or the PackedWeight made from that weight (utils/weight_format.py), here and in the variants below
         - scale_tensor: a fp32 one-item tensor, the product of the two quantisation scales
         - output: an optional (m, n) bfloat16/float16 tensor that is accumulated into: zero-initialised, or
           holding a bias or residual.  Allocated as bfloat16 zeros when omitted.
@@ -91,6 +104,9 @@ def skinny_gemm(
     if output is None:
         output = torch.zeros(size=(skinny_a.size(0), b.size(1)), dtype=torch.bfloat16, device=skinny_a.device)
     skinny_gemm_checks(skinny_a, b, scale_tensor, output)
+    if isinstance(b, PackedWeight):  # the 13-argument op takes the row-major view only
+        _fused(skinny_a, b, output, output, scale_tensor.view(-1), None, None, _capi.EPILOGUE_NONE, 0)
+        return output
     kwargs = infer_skinny_gemm_params(skinny_a, b)
     status = _skinny_gemm(A=skinny_a, B=b, scale_tensor=scale_tensor, D=output, **kwargs)
     _raise_on_status(status, "skinny_gemm_tb")
@@ -114,6 +130,10 @@ def skinny_gemm_scaled(
     skinny_gemm_checks(skinny_a, b, scale_a.reshape(-1)[:1], output)
     assert scale_a.numel() in (1, m) and scale_a.dtype == torch.float32, f"Expected 1 or {m} float32 in scale_a"
     assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
+    if isinstance(b, PackedWeight):
+        _fused(skinny_a, b, output, output if accumulate else None, scale_a.contiguous().view(-1), scale_b.contiguous().view(-1),
+               None, _capi.EPILOGUE_NONE, 0)
+        return output
     status = _skinny_gemm_scaled(skinny_a, b, output, scale_a.contiguous().view(-1), scale_b.contiguous().view(-1),
                                  accumulate)
     _raise_on_status(status, "skinny_gemm_scaled")
@@ -161,8 +181,7 @@ def skinny_gemm_add(
     assert base.shape == output.shape and base.dtype == output.dtype and base.is_contiguous(), (
         f"Expected base to be contiguous with {output.shape = } and {output.dtype = }")
     sa, sb = _scale_vectors(skinny_a, b, scale_a, scale_b)
-    status = _skinny_gemm_fused(skinny_a, b, output, base, sa, sb, None, _capi.EPILOGUE_NONE, 0)
-    _raise_on_status(status, "skinny_gemm_fused")
+    _fused(skinny_a, b, output, base, sa, sb, None, _capi.EPILOGUE_NONE, 0)
     return output
 
 
@@ -200,7 +219,6 @@ def skinny_gemm_swiglu(
     skinny_gemm_checks(skinny_a, gate_up_weight, scale_a.reshape(-1)[:1],
                        _ShapeOnly(m, n, intermediate_dtype, skinny_a.device))
     sa, sb = _scale_vectors(skinny_a, gate_up_weight, scale_a, scale_b)
-    status = _skinny_gemm_fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU,
-                                _capi.BF16 if intermediate_dtype == torch.bfloat16 else _capi.F16)
-    _raise_on_status(status, "skinny_gemm_fused")
+    _fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU,
+           _capi.BF16 if intermediate_dtype == torch.bfloat16 else _capi.F16)
     return output

@@ -14,6 +14,7 @@
 #ifndef HFRK_GFX950_H
 #define HFRK_GFX950_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -42,6 +43,9 @@ enum hfrk_dtype { HFRK_F16 = 0, HFRK_BF16 = 1, HFRK_FP8_E4M3FN = 2 };
 
 /* What happens to the product before it is stored (hfrk_skinny_gemm_fused). */
 enum hfrk_epilogue { HFRK_EPILOGUE_NONE = 0, HFRK_EPILOGUE_SWIGLU = 1 };
+
+/* FP8 flavour of a weight handed to hfrk_pack_weight. */
+enum hfrk_weight_format { HFRK_WEIGHT_E4M3FN = 0, HFRK_WEIGHT_E4M3FNUZ = 1 };
 
 /* Largest m the skinny GEMM accepts. */
 #define HFRK_GEMM_MAX_M 64
@@ -127,6 +131,31 @@ int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scal
 int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
                            const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k,
                            int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
+
+/* Weight load format (no reference counterpart: the reference streams row-major weights through an LDS ring,
+ * csrc/op_src/skinny_gemm/producers/n_full_tiles.cu:4-127, and stores fn bits viewed as fnuz,
+ * hf_rocm_kernels/utils/fp8.py:27-29).  A weight packed once when the model is loaded is read by the GEMM as one
+ * contiguous run per wave, already in matrix-core operand order.
+ *   packed layout: 16-row x 256-byte chunks, rows padded with zeros to a multiple of 16; chunk (tile, kc) at
+ *   (tile * k/256 + kc) * 4096; inside a chunk, 16-byte piece j (0..3) of lane l (0..63) at j*1024 + l*16 holds
+ *   row l%16, bytes (j/2)*128 + (l/16)*32 + (j%2)*16 .. +16.
+ * hfrk_packed_weight_bytes: size of the packed buffer (0 if k % 256 != 0 or a size is not positive).  Host only.
+ * hfrk_pack_weight: src [n,k] fp8 row-major with row stride src_stride -> dst packed.  src_format
+ *   HFRK_WEIGHT_E4M3FNUZ re-encodes on the way (see hfrk_reencode_fnuz).  src and dst must not overlap.
+ * hfrk_unpack_weight: the inverse (padding rows dropped); pack then unpack returns the source bytes.
+ * hfrk_reencode_fnuz: count bytes of e4m3fnuz -> e4m3fn with the same values (dst may be src).  Exact for every
+ *   code except magnitudes below 2^-6, which land on fn's subnormal grid of 2^-9 (round to nearest even); the
+ *   fnuz NaN 0x80 becomes the fn NaN 0x7f.  Scales stay as they are. */
+size_t hfrk_packed_weight_bytes(int n, int k);
+int hfrk_pack_weight(const void* src, int src_stride, int src_format, void* dst, int n, int k, void* stream);
+int hfrk_unpack_weight(const void* src, void* dst, int dst_stride, int n, int k, void* stream);
+int hfrk_reencode_fnuz(const void* src, void* dst, size_t count, void* stream);
+
+/* hfrk_skinny_gemm_fused on a packed weight: same results bit for bit (same operands, same order of sums), B is
+ * the buffer hfrk_pack_weight wrote for this n and k.  With the SwiGLU epilogue n % 32 == 0 as before. */
+int hfrk_skinny_gemm_packed(const void* A, const void* B_packed, void* D, const void* base, const float* scale_a,
+                            int sa_stride, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
+                            int k, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
 
 /* residual <- input + residual (one 16-bit add); output <- rmsnorm(residual) * weight, optionally / scale -> fp8.
  * Replaces `void residual_rms(...)` at csrc/op_src/residual_rms/residual_rms_dispatch.cu:8-63.

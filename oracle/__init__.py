@@ -12,6 +12,7 @@ Modules (each function cites the reference lines it follows):
   residual_rms.py `reference_residual_rms`, `precise_residual_rms`
   swiglu.py       `reference_swiglu`
   llama_mlp.py    the four-op chain
+  weight_format.py packed tile layout (pack / unpack / element offset) and e4m3fnuz -> e4m3fn re-encoding
   c/hfrk_oracle.c plain-C restatement (integer-exact GEMM, scalar RMSNorm/SwiGLU) used to pin the above
 
 How each function is pinned (see tests/test_oracle_*.py):
@@ -22,6 +23,9 @@ How each function is pinned (see tests/test_oracle_*.py):
                   forms (zero, scaled identity, one-hot, powers of two); fp32 path within 1 bf16 ulp of exact
   residual RMS    16-bit add == numpy IEEE add; fp32 path vs fp64 textbook formula; C scalar restatement
   SwiGLU          x*sigmoid(x) closed form == torch.nn.functional.silu; special values; C restatement
+  weight format   fnuz decode table == torch's float8_e4m3fnuz view for all 256 codes and == fn/2 on the same
+                  bits; re-encode table == torch's fnuz -> float -> fn casts for all 256 codes; layout: reshape
+                  implementation == element-offset formula written from the MFMA operand definition, round trip
   llama MLP       composition of the pinned parts; the reference holds no test or fixture for the chain, so
                   the composition itself (which buffer feeds which op) is "parity unpinned" beyond that
 """
