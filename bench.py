@@ -94,9 +94,11 @@ def swiglu_bytes(rows, n):
 
 # ---- GEMM workloads ---------------------------------------------------------------------------------------------------
 
-def make_gemm_inputs(torch, spec):
-    """Activations per (M, K) and len(ms)*cycle quantised copies of each weight, all on the GPU."""
+def make_gemm_inputs(torch, spec, packed=False):
+    """Activations per (M, K) and len(ms)*cycle quantised copies of each weight, all on the GPU (row-major [N, K]
+    passed as the [K, N] view, or -- packed -- converted once to the library's load format)."""
     from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    from hf_rocm_kernels.utils.weight_format import pack_weight
     gen = torch.Generator(device="cuda").manual_seed(0)
     acts, weights = {}, {}
     for m in spec["ms"]:
@@ -116,7 +118,9 @@ def make_gemm_inputs(torch, spec):
         for _ in range(len(spec["ms"]) * spec["cycle"]):
             w = torch.randn((n, k), generator=gen, device="cuda").mul_(0.02)
             sw = amax_scale(w, dim=1) if spec["scaled"] else amax_scale(w)
-            copies.append((fp8_quantize(w, sw)[0].t(), sw.reshape(-1).contiguous()))
+            q = fp8_quantize(w, sw)[0]
+            copies.append((pack_weight(q) if packed else q.t(), sw.reshape(-1).contiguous()))
+            del q
             del w
         weights[name] = copies
     return acts, weights
@@ -259,8 +263,10 @@ def mlp_block_bytes(m):
     return rms_bytes(m, h) + gemm_bytes(m, 2 * inter, h) + swiglu_bytes(m, inter) + gemm_bytes(m, h, inter)
 
 
-def make_mlp_inputs(torch):
+def make_mlp_inputs(torch, packed=False):
     from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    from hf_rocm_kernels.utils.weight_format import pack_weight
+    layout = (lambda q: pack_weight(q)) if packed else (lambda q: q.t())
     gen = torch.Generator(device="cuda").manual_seed(0)
     h, inter = MLP["hidden"], MLP["inter"]
     copies = []
@@ -268,7 +274,7 @@ def make_mlp_inputs(torch):
         wgu = torch.randn((2 * inter, h), generator=gen, device="cuda").mul_(0.02)
         wd = torch.randn((h, inter), generator=gen, device="cuda").mul_(0.02)
         sgu, sd = amax_scale(wgu), amax_scale(wd)
-        copies.append((fp8_quantize(wgu, sgu)[0].t(), sgu.reshape(1), fp8_quantize(wd, sd)[0].t(), sd.reshape(1)))
+        copies.append((layout(fp8_quantize(wgu, sgu)[0]), sgu.reshape(1), layout(fp8_quantize(wd, sd)[0]), sd.reshape(1)))
         del wgu, wd
     acts = {}
     for m in MLP["ms"]:
@@ -377,6 +383,8 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused"], default="llama3-8b")
     ap.add_argument("--detail", action="store_true", help="also time every case on its own (HBM-cold and cache-hot)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--packed", action="store_true",
+                    help="weights in the library's packed load format (hfrk_pack_weight) instead of row-major [N, K]")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed steps run a plain device copy of known size (for scaling rocprofv3 byte counters)")
@@ -391,7 +399,7 @@ def main():
     is_mlp = args.workload in ("mlp", "mlp-fused")
     if is_mlp:
         fused = args.workload == "mlp-fused"
-        copies, acts, rms_w, s_in, s_mid = make_mlp_inputs(torch)
+        copies, acts, rms_w, s_in, s_mid = make_mlp_inputs(torch, args.packed)
         call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused)
         graphs, keep = capture_mlp_steps(torch, call)
         step_bytes = sum(mlp_block_bytes(m) for m in MLP["ms"])
@@ -403,7 +411,7 @@ def main():
         n_copies = MLP["cycle"]
     else:
         spec = WORKLOADS[args.workload]
-        acts, weights = make_gemm_inputs(torch, spec)
+        acts, weights = make_gemm_inputs(torch, spec, args.packed)
         call = gemm_caller(torch, spec, acts, weights)
         graphs, keep = capture_gemm_steps(torch, spec, call)
         n_scales = (lambda m, n: m + n) if spec["scaled"] else (lambda m, n: 1)
@@ -441,10 +449,13 @@ def main():
         "dtype": "fp8_e4m3fn",
         "data": "synthetic",
         "config": {"workload": text, "calls_per_step": calls, "bytes_per_step": step_bytes,
-                   "weight_copies_per_shape": n_copies, "timing": "HIP graph replay, HIP events",
+                   "weight_copies_per_shape": n_copies,
+                   "weight_layout": "packed 16x256-byte chunks in MFMA operand order (hfrk_pack_weight)" if args.packed else "row-major [N, K]",
+                   "timing": "HIP graph replay, HIP events",
                    "us_per_call_mean": round(ms_per_step * 1e3 / calls, 3), "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": None if args.packed else MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
                      "kernel": kernel,
                      "bytes_per_launch": round(step_bytes / calls), "us_per_launch": round(ms_per_step * 1e3 / calls, 3)},
     }

@@ -4,7 +4,7 @@ Counterpart of the reference package's benchmarks/skinny_gemm/grid_search.py, wh
 (a_lanes, b_lanes, qsize, op_m, ops).  Here the search space is `hfrk_gemm_plan`: the wave-stream, K-split and
 workgroup decompositions with their parameters and a few grid sizes, passed to `hfrk_skinny_gemm_ex`.  The rules in
 the library's planner were read off sweeps like this one.  Usage, from the repository root:
-    python hf-rocm-kernels_amd/hf_rocm_kernels/benchmarks/skinny_gemm/grid_search.py -m 8 32 -n 4096 -k 4096 [--json out.json]
+    python hf-rocm-kernels_amd/hf_rocm_kernels/benchmarks/skinny_gemm/grid_search.py -m 8 32 -n 4096 -k 4096 [--packed] [--json out.json]
 """
 import argparse
 import ctypes
@@ -62,18 +62,24 @@ def describe(p: _capi.GemmPlan) -> str:
     return f"workgroup wn={p.wn} wk={p.wk} ch={p.ch} grid={p.grid}"
 
 
-def time_plan(lib, arena: torch.Tensor, m: int, n: int, k: int, plan, reps: int) -> float:
-    """Median microseconds per call from a graph over as many distinct weights as fit the arena (HBM-cold)."""
-    nbuf = max(2, min(64, arena.numel() // (n * k)))
+def time_plan(lib, arena: torch.Tensor, m: int, n: int, k: int, plan, reps: int, packed: bool = False) -> float:
+    """Median microseconds per call from a graph over as many distinct weights as fit the arena (HBM-cold).
+    packed: the arena is read as weights in the packed load format (any bytes are a valid packed weight)."""
+    wbytes = lib.hfrk_packed_weight_bytes(n, k) if packed else n * k
+    nbuf = max(2, min(64, arena.numel() // wbytes))
     a = arena[: m * k]
     scale = torch.ones(1, device=arena.device)
     out = torch.zeros((m, n), dtype=torch.bfloat16, device=arena.device)
-    weights = [arena[i * n * k:(i + 1) * n * k] for i in range(nbuf)]
+    weights = [arena[i * wbytes:(i + 1) * wbytes] for i in range(nbuf)]
     ref = None if plan is None else ctypes.byref(plan)
 
     def call(w: torch.Tensor, stream: int) -> None:
-        status = lib.hfrk_skinny_gemm_ex(a.data_ptr(), w.data_ptr(), out.data_ptr(), scale.data_ptr(), 0, None, 0, m, n, k, k,
-                                         _capi.BF16, 0, ref, stream)
+        if packed:
+            status = lib.hfrk_skinny_gemm_packed(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, scale.data_ptr(), 0, None, 0, None,
+                                                 m, n, k, _capi.BF16, _capi.EPILOGUE_NONE, ref, stream)
+        else:
+            status = lib.hfrk_skinny_gemm_ex(a.data_ptr(), w.data_ptr(), out.data_ptr(), scale.data_ptr(), 0, None, 0, m, n, k, k,
+                                             _capi.BF16, 0, ref, stream)
         if status != 0:
             raise RuntimeError(f"plan rejected with status {status}: {_capi.status_string(status)}")
 
@@ -108,6 +114,7 @@ def main() -> None:
     parser.add_argument("--grids", type=int, nargs="+", default=[256])
     parser.add_argument("--reps", type=int, default=20)
     parser.add_argument("--top", type=int, default=3)
+    parser.add_argument("--packed", action="store_true", help="weights in the packed load format (hfrk_pack_weight)")
     parser.add_argument("--json", default=None, help="write the full table here")
     args = parser.parse_args()
     lib = _capi.load()
@@ -116,11 +123,11 @@ def main() -> None:
     table: Dict[str, dict] = {}
     for m, n, k in itertools.product(args.m, args.n, args.k):
         chosen = _capi.plan(m, n, k)
-        t_default = time_plan(lib, arena, m, n, k, None, args.reps)
+        t_default = time_plan(lib, arena, m, n, k, None, args.reps, args.packed)
         rows = []
         for p in candidate_plans(m, n, k, args.grids):
             try:
-                rows.append((time_plan(lib, arena, m, n, k, p, args.reps), describe(p), p.as_dict()))
+                rows.append((time_plan(lib, arena, m, n, k, p, args.reps, args.packed), describe(p), p.as_dict()))
             except RuntimeError as e:
                 print(f"# {describe(p)}: {e}")
         rows.sort(key=lambda r: r[0])
