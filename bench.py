@@ -16,6 +16,10 @@ Other workloads, same method, for the remaining configurations:
               down GEMM, output added to the residual), hidden 4096, M in {1, 8, 16}: 3 blocks = 12 launches per step
   mlp-fused   the same block in three launches: RMSNorm, gate_up GEMM with SwiGLU epilogue, down GEMM reading the
               residual as its addend (`llama_mlp_combined_ops(..., fused=True)`)
+  pack        the step before the path: the four Llama-3-8B weights packed into the load format from float8_e4m3fn,
+              packed from float8_e4m3fnuz (re-encoded on the way) and unpacked again: 12 launches per step, 2*N*K
+              bytes each (`hf_rocm_kernels.utils.weight_format`)
+`--packed` runs any of the GEMM/MLP workloads on weights in that load format instead of row-major [N, K].
 
 The calls of a step are captured once into a HIP graph (the reference times its kernel the same way,
 operators/skinny_gemm/benchmarking_fn.py:62-92) so the figure is the GPU's, not the Python launch path's.
@@ -375,12 +379,88 @@ def cpu_baseline_mlp(torch, budget_s):
 
 # ---- main -------------------------------------------------------------------------------------------------------------
 
+# ---- weight load format ------------------------------------------------------------------------------------------------
+
+def run_pack_workload(torch, args):
+    """pack (fn source), pack (fnuz source), unpack of the four Llama-3-8B weights; returns the result dict."""
+    from hf_rocm_kernels.utils.weight_format import pack_weight, packed_weight_bytes
+    shapes = WORKLOADS["llama3-8b"]["shapes"]
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    # byte values drawn uniformly: every code of both formats occurs; copies so that no step re-reads cached data
+    copies = 3
+    srcs = {name: [torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda", generator=gen) for _ in range(copies)]
+            for name, n, k in shapes}
+    packed = {name: torch.empty(packed_weight_bytes(n, k), dtype=torch.uint8, device="cuda") for name, n, k in shapes}
+    back = {name: torch.empty((n, k), dtype=torch.uint8, device="cuda") for name, n, k in shapes}
+
+    def run_step(i):
+        for name, n, k in shapes:
+            src = srcs[name][i % copies]
+            torch.ops._HFRK_C.pack_weight(src.view(torch.float8_e4m3fn), packed[name], 0)
+            torch.ops._HFRK_C.unpack_weight(packed[name], back[name])
+            torch.ops._HFRK_C.pack_weight(src.view(torch.float8_e4m3fnuz), packed[name], 1)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        run_step(0)
+    torch.cuda.synchronize()
+    for name, n, k in shapes:  # sanity: the unpacked weight is the source
+        assert torch.equal(back[name], srcs[name][0])
+    graphs = []
+    for i in range(copies):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            run_step(i)
+        graphs.append(g)
+    for i in range(args.warmup):
+        graphs[i % copies].replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(args.steps):
+        graphs[i % copies].replay()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    step_bytes = sum(3 * 2 * n * k for _, n, k in shapes)
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    calls = 3 * len(shapes)
+    result = {
+        "metric": "weight load format: pack / re-encoding pack / unpack of the Llama-3-8B weights, achieved HBM GB/s",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "pack (e4m3fn), unpack, pack (e4m3fnuz -> e4m3fn) of qkv(6144,4096) o_proj(4096,4096) "
+                               "gate_up(28672,4096) down(4096,14336); 12 launches per step, read N*K + write N*K bytes each",
+                   "calls_per_step": calls, "bytes_per_step": step_bytes, "timing": "HIP graph replay, HIP events"},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "hfrk::pack_weight_kernel<UNPACK,FNUZ>",
+                     "bytes_per_launch": round(step_bytes / calls), "us_per_launch": round(ms_per_step * 1e3 / calls, 3)},
+    }
+    del graphs
+    if not args.no_cpu:
+        from oracle import weight_format as wf
+        import numpy as np
+        t_all, moved = [], 0
+        for name, n, k in shapes[:2]:  # the two small weights bound the CPU leg to a few seconds
+            w = srcs[name][0].cpu().numpy()
+            t0 = time.perf_counter()
+            p = wf.pack_weight(w)
+            wf.unpack_weight(p, n, k)
+            wf.pack_weight(wf.reencode_fnuz(w))
+            t_all.append(time.perf_counter() - t0)
+            moved += 3 * 2 * n * k
+        result["cpu_baseline"] = {"value": round(moved / sum(t_all) / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                                  "sample": "oracle numpy pack / unpack / re-encoding pack of the qkv and o_proj weights, one pass"}
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused"], default="llama3-8b")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "pack"], default="llama3-8b")
     ap.add_argument("--detail", action="store_true", help="also time every case on its own (HBM-cold and cache-hot)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--packed", action="store_true",
@@ -396,6 +476,9 @@ def main():
         sys.exit("bench.py needs a GPU (the kernels have no CPU path)")
     torch.cuda.set_device(0)
 
+    if args.workload == "pack":
+        print(json.dumps(run_pack_workload(torch, args)))
+        return
     is_mlp = args.workload in ("mlp", "mlp-fused")
     if is_mlp:
         fused = args.workload == "mlp-fused"
