@@ -1,6 +1,8 @@
-// Per-token (per-row) dynamic FP8 quantisation fused into the two element-wise kernels of the decoder block:
+// Per-token (per-row) dynamic FP8 quantisation fused into the two element-wise kernels of the decoder block, and on
+// its own for activations that come from elsewhere (attention output -> o_proj):
 //   residual_rms_dynamic:  residual <- input + residual;  y = rmsnorm(residual) * weight
 //   swiglu_dynamic:        y = silu(gate) * up
+//   quantize_fp8:          y = x   (also with one static scale: the reference's fp8_quantize, utils/fp8.py:6-29, on device)
 // and in both:            scale[row] = max(amax_row |y| / 448, FLT_MIN);  output = e4m3fn(y / scale[row])
 // The per-row scales feed the GEMM's per-token scale_a directly, so no activation scale has to be calibrated ahead
 // of time.  The reference only has the static-scale forms (one scale_tensor for the whole tensor:
@@ -173,6 +175,53 @@ __global__ void __launch_bounds__(kDynMaxThreads) swiglu_dynamic_kernel(
     dyn_zero_row(next_buffer, buffer_cols);
 }
 
+// Plain quantisation of a 16-bit activation block (what sits between an attention output and the o_proj GEMM):
+// dynamic (static_scale == nullptr): scales[row] = max(amax_row |x| / 448, FLT_MIN), output = e4m3fn(x / scales[row]);
+// static: output = e4m3fn(x / static_scale[0]), saturating, scales untouched.
+template <int DT, int ITERS>
+__global__ void __launch_bounds__(kDynMaxThreads) quantize_rows_kernel(
+    const uint16_t* __restrict__ input, const float* __restrict__ static_scale, uint8_t* __restrict__ output,
+    float* __restrict__ scales, int cols) {
+    __shared__ float red_max[16];
+    const uint16_t* const row = input + (long)blockIdx.x * cols;
+    const int nvec = cols >> 3;
+    float y[ITERS][8];
+    float amax = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = threadIdx.x + it * blockDim.x;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[it][j] = 0.f;
+        if (v < nvec) {
+            const v4i x = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row) + v);
+            const uint32_t xw[4] = {(uint32_t)x[0], (uint32_t)x[1], (uint32_t)x[2], (uint32_t)x[3]};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                y[it][2 * j] = load16<DT>((uint16_t)(xw[j] & 0xffff));
+                y[it][2 * j + 1] = load16<DT>((uint16_t)(xw[j] >> 16));
+                amax = fmaxf(amax, fmaxf(fabsf(y[it][2 * j]), fabsf(y[it][2 * j + 1])));
+            }
+        }
+    }
+    if (static_scale) {
+        const float inv = 1.0f / static_scale[0];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int v = threadIdx.x + it * blockDim.x;
+            if (v < nvec) {
+                uint32_t p0 = cvt_pk_fp8(y[it][0] * inv, y[it][1] * inv, 0u, false);
+                p0 = cvt_pk_fp8(y[it][2] * inv, y[it][3] * inv, p0, true);
+                uint32_t p1 = cvt_pk_fp8(y[it][4] * inv, y[it][5] * inv, 0u, false);
+                p1 = cvt_pk_fp8(y[it][6] * inv, y[it][7] * inv, p1, true);
+                reinterpret_cast<uint2*>(output + (long)blockIdx.x * cols)[v] = make_uint2(p0, p1);
+            }
+        }
+        return;
+    }
+    amax = dyn_block_max(amax, red_max);
+    dyn_quantise_row<ITERS>(y, amax, output + (long)blockIdx.x * cols, scales, nvec);
+}
+
 static bool dyn_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // threads and register-cache depth for a row of `nvec` 16-byte pieces; false when the row does not fit
@@ -246,6 +295,31 @@ extern "C" int hfrk_swiglu_dynamic(const void* gate_up, void* output, float* sca
         if (iters == 1) HFRK_DYN_SWIGLU(HFRK_BF16, 1); else if (iters == 2) HFRK_DYN_SWIGLU(HFRK_BF16, 2); else HFRK_DYN_SWIGLU(HFRK_BF16, 4);
     }
 #undef HFRK_DYN_SWIGLU
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}
+
+extern "C" int hfrk_quantize_fp8(const void* input, const float* static_scale, void* output, float* scales, int rows, int cols,
+                                 int io_dtype, void* stream) {
+    using namespace hfrk;
+    if (rows < 0 || cols < 1 || cols % 8 != 0) return HFRK_BAD_SHAPE;
+    if (rows == 0) return HFRK_SUCCESS;
+    if (!input || !output || (!static_scale && !scales)) return HFRK_BAD_SHAPE;
+    if (io_dtype != HFRK_F16 && io_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
+    if (!dyn_aligned16(input) || (reinterpret_cast<uintptr_t>(output) & 7)) return HFRK_BAD_ALIGNMENT;
+    int threads = 0, iters = 0;
+    if (!dyn_geometry(cols / 8, &threads, &iters)) return HFRK_BAD_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint16_t* in = static_cast<const uint16_t*>(input);
+    uint8_t* out = static_cast<uint8_t*>(output);
+#define HFRK_QUANT(DT_, IT_) \
+    hipLaunchKernelGGL((quantize_rows_kernel<DT_, IT_>), dim3(rows), dim3(threads), 0, s, in, static_scale, out, scales, cols)
+    if (io_dtype == HFRK_F16) {
+        if (iters == 1) HFRK_QUANT(HFRK_F16, 1); else if (iters == 2) HFRK_QUANT(HFRK_F16, 2); else HFRK_QUANT(HFRK_F16, 4);
+    } else {
+        if (iters == 1) HFRK_QUANT(HFRK_BF16, 1); else if (iters == 2) HFRK_QUANT(HFRK_BF16, 2); else HFRK_QUANT(HFRK_BF16, 4);
+    }
+#undef HFRK_QUANT
     HFRK_HIP_TRY(hipGetLastError());
     return HFRK_SUCCESS;
 }

@@ -233,6 +233,32 @@ void swiglu_dynamic(at::Tensor& gate_up, at::Tensor& output, at::Tensor& scales,
              "swiglu_dynamic");
 }
 
+// 16-bit [rows, cols] -> float8_e4m3fn: with one static scale (the reference's fp8_quantize, hf_rocm_kernels/utils/fp8.py:6-29,
+// as one kernel) or, scale_tensor None, one dynamic scale per row written to `scales`.
+void quantize_fp8(at::Tensor& input, const std::optional<at::Tensor>& scale_tensor, at::Tensor& output, at::Tensor& scales) {
+    TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous [rows, cols] tensor");
+    const int io = dtype16(input, "input");
+    check_fp8(output, "output");
+    TORCH_CHECK(output.sizes() == input.sizes() && output.is_contiguous(), "output must match input and be contiguous");
+    check_same_device(input, output, "output");
+    const float* static_scale = nullptr;
+    float* scales_ptr = nullptr;
+    if (scale_tensor.has_value()) {
+        TORCH_CHECK(scale_tensor->numel() == 1 && scale_tensor->scalar_type() == at::kFloat, "scale_tensor must be one float32");
+        check_same_device(input, *scale_tensor, "scale_tensor");
+        static_scale = scale_tensor->data_ptr<float>();
+    } else {
+        TORCH_CHECK(scales.scalar_type() == at::kFloat && scales.is_contiguous() && scales.numel() == input.size(0),
+                    "scales must be a contiguous float32 tensor with one element per row");
+        check_same_device(input, scales, "scales");
+        scales_ptr = scales.data_ptr<float>();
+    }
+    DeviceScope scope(input);
+    raise_on(hfrk_quantize_fp8(input.data_ptr(), static_scale, output.data_ptr(), scales_ptr, (int)input.size(0), (int)input.size(1), io,
+                               current_stream(input)),
+             "quantize_fp8");
+}
+
 // The GEMM with the surrounding element-wise work folded in.  No reference counterpart as one op.
 //   epilogue 0: D = (base ? base : 0) + scale_a x scale_b x A.B, base a 16-bit [m,n] tensor (D itself, a residual) or None
 //   epilogue 1: B is a gate_up weight [k, 2*inter]; D fp8 [m, inter] = e4m3fn(silu(gate) * up / out_scale), the two
@@ -400,6 +426,9 @@ TORCH_LIBRARY(_HFRK_C, ops) {
 
     ops.def("swiglu_dynamic(Tensor gate_up, Tensor! output, Tensor! scales, Tensor! next_buffer) -> ()");
     ops.impl("swiglu_dynamic", c10::kCUDA, &swiglu_dynamic);
+
+    ops.def("quantize_fp8(Tensor input, Tensor? scale_tensor, Tensor! output, Tensor! scales) -> ()");
+    ops.impl("quantize_fp8", c10::kCUDA, &quantize_fp8);
 }
 
 // `import hf_rocm_kernels._HFRK_C` loads this library and thereby runs the registration above.

@@ -8,6 +8,7 @@ from .operators.increment import increment
 from .operators.residual_rms import residual_rms, residual_rms_dynamic
 from .operators.swiglu import swiglu, swiglu_dynamic
 from .operators.skinny_gemm import skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu
+from .operators.quantize import quantize_fp8
 
 __all__ = ["increment", "residual_rms", "swiglu", "skinny_gemm", "skinny_gemm_scaled", "skinny_gemm_add",
-           "skinny_gemm_swiglu", "residual_rms_dynamic", "swiglu_dynamic"]
+           "skinny_gemm_swiglu", "residual_rms_dynamic", "swiglu_dynamic", "quantize_fp8"]

@@ -70,6 +70,7 @@ SIGNATURES = {
     "hfrk_swiglu": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "hfrk_residual_rms_dynamic": (_i, [_p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _p]),
     "hfrk_swiglu_dynamic": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "hfrk_quantize_fp8": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
 }
 
 _lib = None

@@ -1,0 +1,112 @@
+"""Linear-layer front end of the FP8 skinny GEMM: what a serving stack binds in place of its fp8 linear method.
+
+The reference points to its vLLM integration for this (README.md:95-97); the hook there replaces the fp8 linear
+apply function for decode-sized batches.  This module is that hook without the vLLM dependency: a function with the
+usual (input, weight, weight_scale, input_scale, bias) signature, and an nn.Module that owns a quantised weight.
+
+Decode batches (up to 64 tokens) run as: one quantisation kernel (skipped when the caller already holds fp8
+activations and their scales, e.g. from `residual_rms_dynamic` / `swiglu_dynamic`) and one GEMM with the scales, the
+bias or residual folded into its epilogue.  Larger batches are cut into pieces of 64 rows; a prefill-sized batch
+belongs on a GEMM library and is only handled here so that the layer is always correct.
+"""
+from typing import Optional, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from .. import _capi
+from ..operators.quantize import quantize_fp8
+from ..operators.skinny_gemm import skinny_gemm_add, skinny_gemm_scaled
+from ..utils.fp8 import amax_scale, fp8_quantize
+from ..utils.weight_format import PackedWeight, pack_weight
+
+Weight = Union[Tensor, PackedWeight]
+
+
+def _weight_view(weight: Weight) -> Weight:
+    """[n, k] row-major fp8 (an nn.Linear weight) -> the [k, n] view the GEMM takes; a PackedWeight passes through."""
+    return weight if isinstance(weight, PackedWeight) else weight.t()
+
+
+def apply_fp8_linear(
+    input: Tensor,
+    weight: Weight,
+    weight_scale: Tensor,
+    input_scale: Optional[Tensor] = None,
+    bias: Optional[Tensor] = None,
+    residual: Optional[Tensor] = None,
+    out_dtype: Optional[torch.dtype] = None,
+) -> Tensor:
+    """y = input @ dequant(weight).T (+ bias) (+ residual), computed in FP8 with fp32 accumulation.
+
+    - input: (..., k) float16/bfloat16 activations, quantised here -- with `input_scale` (one float32: static) or,
+      when it is None, dynamically per token -- or a float8_e4m3fn tensor already quantised, `input_scale` then being
+      its scale(s): one float32 or one per token
+    - weight: (n, k) float8_e4m3fn row-major, or its PackedWeight; weight_scale: one float32 or one per output channel
+    - bias: (n,) in the output dtype; residual: (..., n) in the output dtype, added in the GEMM's epilogue (fp32 sum
+      with the product, one rounding).  Given both, the bias is added to the residual first (one 16-bit add).
+    - out_dtype: float16/bfloat16; defaults to the input's (bfloat16 for an fp8 input)
+    """
+    k = input.shape[-1]
+    lead = input.shape[:-1]
+    x = input.reshape(-1, k)
+    if x.dtype == torch.float8_e4m3fn:
+        assert input_scale is not None, "an fp8 input needs its scale(s)"
+        q, sa = x.contiguous(), input_scale.reshape(-1)
+        out_dtype = out_dtype or torch.bfloat16
+    else:
+        out_dtype = out_dtype or x.dtype
+        q, sa = quantize_fp8(x.contiguous(), input_scale)
+        sa = sa.reshape(-1)
+    w = _weight_view(weight)
+    n = w.size(1)
+    sb = weight_scale.reshape(-1)
+    m = q.size(0)
+    base = None
+    if residual is not None:
+        base = residual.reshape(m, n)
+        if bias is not None:
+            base = base + bias
+        base = base.contiguous()
+    elif bias is not None:
+        base = bias.to(out_dtype).expand(m, n).contiguous()
+    out = torch.empty((m, n), dtype=out_dtype, device=q.device)
+    for r0 in range(0, m, _capi.GEMM_MAX_M):
+        r1 = min(m, r0 + _capi.GEMM_MAX_M)
+        sa_part = sa if sa.numel() == 1 else sa[r0:r1]
+        if base is None:
+            skinny_gemm_scaled(q[r0:r1], w, sa_part, sb, output=out[r0:r1])
+        else:
+            skinny_gemm_add(q[r0:r1], w, sa_part, sb, base[r0:r1], output=out[r0:r1])
+    return out.reshape(*lead, n)
+
+
+class Fp8Linear(torch.nn.Module):
+    """nn.Linear with an FP8 weight: per-output-channel (default) or per-tensor weight scale, dynamic per-token or
+    static activation scale, optional packed load format.  Inference only."""
+
+    def __init__(self, weight: Weight, weight_scale: Tensor, bias: Optional[Tensor] = None,
+                 input_scale: Optional[Tensor] = None):
+        super().__init__()
+        self.weight, self.weight_scale, self.bias, self.input_scale = weight, weight_scale, bias, input_scale
+        self.out_features, self.in_features = (weight.n, weight.k) if isinstance(weight, PackedWeight) else tuple(weight.shape)
+
+    @classmethod
+    def from_float(cls, linear: torch.nn.Linear, per_channel: bool = True, packed: bool = False,
+                   input_scale: Optional[Tensor] = None) -> "Fp8Linear":
+        """Quantise an nn.Linear's weight (scale = amax/448 per output channel or per tensor)."""
+        w = linear.weight.detach()
+        scale = amax_scale(w, dim=1 if per_channel else None)
+        q, _ = fp8_quantize(w, scale)
+        weight = pack_weight(q) if packed else q
+        bias = None if linear.bias is None else linear.bias.detach()
+        return cls(weight, scale.reshape(-1).contiguous(), bias, input_scale)
+
+    def forward(self, input: Tensor, input_scale: Optional[Tensor] = None, residual: Optional[Tensor] = None) -> Tensor:
+        """`input` 16-bit (quantised here) or fp8 with `input_scale`; `residual` is added in the GEMM's epilogue."""
+        scale = input_scale if input_scale is not None else self.input_scale
+        return apply_fp8_linear(input, self.weight, self.weight_scale, scale, self.bias, residual)
+
+    def extra_repr(self) -> str:
+        kind = "packed" if isinstance(self.weight, PackedWeight) else "row-major"
+        return f"in_features={self.in_features}, out_features={self.out_features}, weight={kind}, bias={self.bias is not None}"

@@ -187,6 +187,14 @@ int hfrk_residual_rms_dynamic(const void* input, void* residual, const void* wei
 int hfrk_swiglu_dynamic(const void* gate_up, void* output, float* scales, void* next_buffer, int rows, int cols,
                         int buffer_cols, int io_dtype, void* stream);
 
+/* FP8 quantisation of a 16-bit activation block [rows, cols] (the device form of fp8_quantize,
+ * hf_rocm_kernels/utils/fp8.py:6-29, which the reference runs as torch ops on the caller's side; here also per token).
+ *   static_scale != NULL:  output = e4m3fn(clamp(input / static_scale[0], +-448)); scales is not touched (may be NULL)
+ *   static_scale == NULL:  scales[r] = max(amax_c |input[r,c]| / 448, FLT_MIN); output[r,c] = e4m3fn(input[r,c] / scales[r])
+ * Same limits as the dynamic kernels above: cols % 8 == 0, cols <= 32768, 16-byte aligned input, 8-byte aligned output. */
+int hfrk_quantize_fp8(const void* input, const float* static_scale, void* output, float* scales, int rows, int cols,
+                      int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
