@@ -28,6 +28,7 @@
 //    results are bit-reproducible -- applies the scales once, adds D (accumulate mode) and rounds once.
 #include <mutex>
 #include <type_traits>
+#include <unordered_map>
 
 #include "skinny_gemm_args.h"
 
@@ -633,6 +634,32 @@ static int launch_mt(const GemmArgs& args, const hfrk_gemm_plan& p, hipStream_t 
     return HFRK_INVALID_CONFIG;
 }
 
+// ---- plan table: tuned decompositions that replace the planner's rule for exact (m, n, k, weight layout) keys ----------
+// Filled by an autotuner (hfrk_plan_table_set) from on-device sweeps; consulted whenever a caller leaves the plan to
+// the library.  Counterpart of the reference's tuned knob table (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102).
+static std::unordered_map<uint64_t, hfrk_gemm_plan> g_plan_table;
+static std::mutex g_plan_mutex;
+
+static bool plan_key(int m, int n, int k, int packed, uint64_t* key) {
+    if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || n >= (1 << 24) || k < 1 || (k >> 8) >= (1 << 16) || k % 256 != 0) return false;
+    *key = ((uint64_t)(packed ? 1 : 0) << 47) | ((uint64_t)m << 40) | ((uint64_t)n << 16) | (uint64_t)(k >> 8);
+    return true;
+}
+
+// the tuned plan if there is one, else the planner's
+static int choose_plan(int m, int n, int k, bool packed, hfrk_gemm_plan* plan) {
+    uint64_t key;
+    if (plan_key(m, n, k, packed, &key)) {
+        std::lock_guard<std::mutex> lock(g_plan_mutex);
+        const auto it = g_plan_table.find(key);
+        if (it != g_plan_table.end()) {
+            *plan = it->second;
+            return HFRK_SUCCESS;
+        }
+    }
+    return make_plan(m, n, k, plan);
+}
+
 // D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
 static int gemm_launch(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
                        const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k, int b_stride,
@@ -663,7 +690,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         const int rc = check_plan(m, swiglu ? n / 2 : n, k, swiglu, &p);
         if (rc != HFRK_SUCCESS) return rc;
     } else {
-        const int rc = swiglu ? fill_stream_plan(m, n / 2, k, 1, false, 0, &p) : make_plan(m, n, k, &p);
+        const int rc = swiglu ? fill_stream_plan(m, n / 2, k, 1, false, 0, &p) : choose_plan(m, n, k, packed, &p);
         if (rc != HFRK_SUCCESS) return rc;
         if (swiglu) {  // same chunk count as a one-tile plan over n/2 rows, but every chunk holds a gate and an up tile
             p.wk = 2;
@@ -745,6 +772,31 @@ int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, in
 int hfrk_skinny_gemm_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (!plan) return HFRK_BAD_SHAPE;
     return hfrk::make_plan(m, n, k, plan);
+}
+
+int hfrk_plan_table_set(int m, int n, int k, int packed, const hfrk_gemm_plan* plan) {
+    uint64_t key;
+    if (!hfrk::plan_key(m, n, k, packed, &key)) return HFRK_BAD_SHAPE;
+    if (plan) {
+        const int rc = hfrk::check_plan(m, n, k, false, plan);
+        if (rc != HFRK_SUCCESS) return rc;
+    }
+    std::lock_guard<std::mutex> lock(hfrk::g_plan_mutex);
+    if (plan) hfrk::g_plan_table[key] = *plan;
+    else hfrk::g_plan_table.erase(key);
+    return HFRK_SUCCESS;
+}
+
+int hfrk_plan_table_get(int m, int n, int k, int packed, hfrk_gemm_plan* plan) {
+    if (!plan) return HFRK_BAD_SHAPE;
+    return hfrk::choose_plan(m, n, k, packed != 0, plan);
+}
+
+int hfrk_plan_table_clear(void) {
+    std::lock_guard<std::mutex> lock(hfrk::g_plan_mutex);
+    const int size = (int)hfrk::g_plan_table.size();
+    hfrk::g_plan_table.clear();
+    return size;
 }
 
 int hfrk_skinny_gemm(const void* A, const void* B, void* D, const float* scale_tensor, int m, int n, int k,

@@ -58,6 +58,9 @@ SIGNATURES = {
     "hfrk_status_string": (ctypes.c_char_p, [_i]),
     "hfrk_skinny_gemm_validate": (_i, [_i] * 13),
     "hfrk_skinny_gemm_plan": (_i, [_i, _i, _i, ctypes.POINTER(GemmPlan)]),
+    "hfrk_plan_table_set": (_i, [_i, _i, _i, _i, ctypes.POINTER(GemmPlan)]),
+    "hfrk_plan_table_get": (_i, [_i, _i, _i, _i, ctypes.POINTER(GemmPlan)]),
+    "hfrk_plan_table_clear": (_i, []),
     "hfrk_skinny_gemm": (_i, [_p, _p, _p, _p] + [_i] * 14 + [_p]),
     "hfrk_skinny_gemm_ex": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),

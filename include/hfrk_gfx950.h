@@ -95,6 +95,18 @@ int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, in
  * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102).  Returns HFRK_SUCCESS or a shape error. */
 int hfrk_skinny_gemm_plan(int m, int n, int k, hfrk_gemm_plan* plan);
 
+/* Plan table (host only, thread-safe): tuned decompositions that take the planner's place for exact keys
+ * (m, n, k, packed) whenever a GEMM entry point is called without a plan (the SwiGLU epilogue keeps its own plan).
+ * Counterpart of the reference's tuned table, hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102, filled from
+ * sweeps like its benchmarks/skinny_gemm/grid_search.py.
+ *   hfrk_plan_table_set    validates the plan for the shape like hfrk_skinny_gemm_ex does and stores it; plan == NULL
+ *                          removes the entry.  Returns HFRK_SUCCESS or the validation status.
+ *   hfrk_plan_table_get    the plan a call without one would use: the entry, or the planner's choice.
+ *   hfrk_plan_table_clear  drops every entry, returns how many there were. */
+int hfrk_plan_table_set(int m, int n, int k, int packed, const hfrk_gemm_plan* plan);
+int hfrk_plan_table_get(int m, int n, int k, int packed, hfrk_gemm_plan* plan);
+int hfrk_plan_table_clear(void);
+
 /* D[m,n] += scale_tensor[0] * A[m,k] . B[k,n]
  * Replaces `int skinny_gemm(...)` at csrc/op_src/skinny_gemm/skinny_gemm_caller.cu:21-32, the function behind
  * torch.ops._HFRK_C.skinny_gemm_tb (csrc/op_src/skinny_gemm/skinny_gemm_binding.cu:16-42), same argument order.

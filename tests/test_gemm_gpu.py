@@ -401,3 +401,31 @@ def test_benchmarking_helpers_and_the_library_gemm_agree_with_scaled_mm():
     bench = Bench()
     bench.add_measure("add", 1024, lambda: torch.zeros(1024, device="cuda").add_(1), rep=4)
     assert bench.table("n")["add"][0] > 0
+
+
+def test_a_plan_table_entry_is_what_a_call_without_a_plan_runs():
+    """An entry that moves m = 8 to the workgroup kernel with an odd grid: the default call then gives, bit for bit,
+    what the explicit plan gives, on the row-major and on the packed key, and the oracle's answer."""
+    from hf_rocm_kernels import plan_table, skinny_gemm_scaled
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    from hf_rocm_kernels.utils.weight_format import pack_weight
+    m, n, k = 8, 2048, 4096
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=21)
+    entry = _capi.GemmPlan(1, 2, 4, 1, 23, n // 32, k // 1024, 8 * 4096 + 2 * 16 * 1024 + 16)
+    explicit = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    run_ex(a, b, sa, sw, explicit, accumulate=False, plan=entry)
+    plan_table.clear()
+    try:
+        before = skinny_gemm_scaled(a, b, sa, sw)
+        plan_table.set_plan(m, n, k, entry)
+        plan_table.set_plan(m, n, k, entry, packed=True)
+        assert plan_table.get_plan(m, n, k).as_dict() == entry.as_dict()
+        after = skinny_gemm_scaled(a, b, sa, sw)
+        after_packed = skinny_gemm_scaled(a, pack_weight(b.t()), sa, sw)
+    finally:
+        plan_table.clear()
+        plan_table.load_from_environment()
+    assert torch.equal(after, explicit) and torch.equal(after_packed, explicit)
+    check_against_oracle(after, a, b, sa, sw)
+    check_against_oracle(before, a, b, sa, sw)

@@ -307,3 +307,61 @@ def test_bench_table_bookkeeping():
     x = torch.zeros(4, 4, dtype=torch.float16)
     y = randomize_tensors(x)
     assert y.shape == x.shape and y.dtype == x.dtype and not torch.equal(x, y) and randomize_tensors(3) == 3
+
+
+def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_path, monkeypatch):
+    """hfrk_plan_table_* are host functions: entries replace the planner's choice for their exact key, invalid plans
+    are refused with the launcher's status, and a table survives save -> clear -> load (also via HFRK_PLAN_TABLE)."""
+    from hf_rocm_kernels import plan_table
+    plan_table.clear()
+    m, n, k = 8, 6144, 4096
+    planner = _capi.plan(m, n, k)
+    assert plan_table.get_plan(m, n, k).as_dict() == planner.as_dict()
+    tuned = _capi.GemmPlan(1, 0, 1, 2, 128, planner.panels, planner.slabs, planner.lds_bytes)  # same kernel, grid 128
+    assert tuned.as_dict() != planner.as_dict()
+    plan_table.set_plan(m, n, k, tuned)
+    assert plan_table.get_plan(m, n, k).as_dict() == tuned.as_dict()
+    assert _capi.plan(m, n, k).as_dict() == planner.as_dict()          # hfrk_skinny_gemm_plan stays the planner's rule
+    assert plan_table.get_plan(m, n, k, packed=True).as_dict() == planner.as_dict()   # another key
+    assert plan_table.get_plan(m + 1, n, k).as_dict() == _capi.plan(m + 1, n, k).as_dict()
+    # a plan that does not fit the shape is refused and changes nothing
+    bad = _capi.GemmPlan(1, 0, 1, 1, 128, planner.panels, planner.slabs, planner.lds_bytes)  # 4 rows of activations for m = 8
+    with pytest.raises(RuntimeError):
+        plan_table.set_plan(m, n, k, bad)
+    assert _capi.load().hfrk_plan_table_set(m, n, 100, 0, ctypes.byref(tuned)) == _capi.BAD_SHAPE
+    assert plan_table.get_plan(m, n, k).as_dict() == tuned.as_dict()
+    # a workgroup-kernel entry for a shape the planner gives to the wave-stream kernel
+    wg = _capi.GemmPlan(1, 4, 2, 1, 200, n // 64, k // 512, 8 * 4096 + 2 * 16 * 512 + 16)
+    plan_table.set_plan(16, n, k, wg, packed=True)
+    path = tmp_path / "table.json"
+    plan_table.save([{"m": m, "n": n, "k": k, "packed": False, "plan": tuned.as_dict(), "us": 7.5},
+                     {"m": 16, "n": n, "k": k, "packed": True, "plan": wg.as_dict()}], str(path))
+    assert plan_table.clear() == 2
+    assert plan_table.get_plan(m, n, k).as_dict() == planner.as_dict()
+    assert plan_table.load(str(path)) == 2
+    assert plan_table.get_plan(m, n, k).as_dict() == tuned.as_dict()
+    assert plan_table.get_plan(16, n, k, packed=True).as_dict() == wg.as_dict()
+    plan_table.remove_plan(m, n, k)
+    assert plan_table.get_plan(m, n, k).as_dict() == planner.as_dict()
+    assert plan_table.clear() == 1
+    monkeypatch.setenv(plan_table.ENV_VAR, str(path))
+    assert plan_table.load_from_environment() == 2
+    assert plan_table.clear() == 2
+    monkeypatch.setenv(plan_table.ENV_VAR, "none")
+    assert plan_table.load_from_environment() is None
+    monkeypatch.delenv(plan_table.ENV_VAR)
+    shipped = plan_table.load_from_environment()   # the table shipped with the package: every entry must be accepted
+    import json
+    assert shipped == len(json.load(open(plan_table.DEFAULT_TABLE))["entries"]) and shipped > 0
+    assert plan_table.clear() == shipped
+    other = tmp_path / "other.json"
+    other.write_text('{"format": "something else", "entries": []}')
+    with pytest.raises(ValueError):
+        plan_table.load(str(other))
+    # an entry the library rejects: strict raises, non-strict skips it
+    plan_table.save([{"m": m, "n": n, "k": k, "plan": bad.as_dict()}, {"m": m, "n": n, "k": k, "plan": tuned.as_dict()}], str(other))
+    with pytest.raises(RuntimeError):
+        plan_table.load(str(other))
+    plan_table.clear()
+    assert plan_table.load(str(other), strict=False) == 1
+    plan_table.clear()
