@@ -48,8 +48,8 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
 
 HBM_PEAK_GBPS = 8000.0
 # Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised in profiles/skinny_gemm_stream_llama3_8b_decode_hbm_traffic.txt: 1.0096 x the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55223910}
+# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0099 x the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55240479}
 CALIBRATION_COPY_BYTES = 256 << 20
 
 WORKLOADS = {
@@ -59,7 +59,8 @@ WORKLOADS = {
         "text": "llama3-8b decode linears: M in {1,2,4,8,16} x qkv(6144,4096) o_proj(4096,4096) gate_up(28672,4096) "
                 "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-8B decode shapes, M=1..16 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel<MA,RT> (all 20 launches of a step)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel (16 of the 20 launches of a step); with the shipped plan table "
+                  "hfrk::skinny_gemm_kernel<1,8,1,2> on gate_up at M=1,8,16 and hfrk::skinny_gemm_ksplit_kernel<1,512> on qkv at M=16",
     },
     "llama3-70b": {
         "shapes": [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)],
@@ -67,7 +68,8 @@ WORKLOADS = {
         "text": "llama3-70b decode linears: M in {1,4,8,16,32} x qkv(10240,8192) o_proj(8192,8192) gate_up(57344,8192) "
                 "down(8192,28672); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-70B decode shapes, M=1..32 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel<MA,RT> (M<=16), hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel (M<=8), stream / workgroup kernel by plan table (M=16), "
+                  "hfrk::skinny_gemm_kernel / skinny_gemm_ksplit_kernel (M=32)",
     },
     "scaled-m": {
         "shapes": [("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)],
@@ -75,7 +77,8 @@ WORKLOADS = {
         "text": "M in {16,32,64} x (4096,4096) (28672,4096) (4096,14336); FP8 e4m3fn, per-token activation scales "
                 "(rows 1 and M-1 are 20x outliers) and per-output-channel weight scales, bf16 out; 9 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s, per-token x per-channel scales, M=16..64 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel<4,RT> (M=16), hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel / skinny_gemm_kernel (M=16), hfrk::skinny_gemm_ksplit_kernel (M=32,64 on K=4096), "
+                  "hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64 on K=14336 and plan-table entries)",
     },
 }
 MLP = {"hidden": 4096, "inter": 14336, "ms": [1, 8, 16], "cycle": 12, "eps": 1e-5,
