@@ -171,10 +171,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     v4i aq[APT];
     // always called just before issue_unit for the same unit, so (ip, is) name that unit
     auto act_load = [&](bool in_range) __attribute__((always_inline)) {
-        uint32_t base = in_range ? (uint32_t)phys_slab(ip, is) * KS : 0x80000000u;
-#ifdef HFRK_EXP_NOACT  // measurement only: request nothing, results are wrong
-        base = 0x80000000u;
-#endif
+        const uint32_t base = in_range ? (uint32_t)phys_slab(ip, is) * KS : 0x80000000u;
 #pragma unroll
         for (int q = 0; q < APT; ++q) {
             const int idx = tid + q * kGemmThreads;
