@@ -78,18 +78,29 @@ class Bench:
         return metrics
 
     @classmethod
-    def benchmark_fn(cls, fn: Callable[[], None], rep: int = 100, warmup: int = 10, graph_size: int = 8) -> float:
-        """Median microseconds per call of fn() from `rep` replays of a graph of `graph_size` calls."""
+    def benchmark_fn(cls, fn: Callable[[], None], rep: int = 100, warmup: int = 10, graph_size: int = 0) -> float:
+        """Median microseconds per call of fn() from `rep` replays of a graph of `graph_size` calls.
+        graph_size 0 sizes the graph from a first estimate so that one replay lasts about a millisecond (8 to 256
+        calls): launching a graph costs some ten microseconds however small it is, which a graph of a few
+        microsecond-sized kernels would otherwise report as kernel time (the reference gets the same effect from
+        triton's do_bench_cudagraph, utils/benchmarking.py:60-75)."""
         stream = torch.cuda.Stream()
+
+        def capture(calls: int) -> "torch.cuda.CUDAGraph":
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for _ in range(calls):
+                    fn()
+            torch.cuda.synchronize()
+            return graph
+
         with torch.cuda.stream(stream):
             fn()
             torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                for _ in range(graph_size):
-                    fn()
-            torch.cuda.synchronize()
-            samples = sorted(_time_graph_replays(graph, graph_size, max(warmup, 0), rep))
+            if graph_size <= 0:
+                probe = sorted(_time_graph_replays(capture(8), 8, 2, 5))
+                graph_size = int(min(256, max(8, 1000.0 / max(probe[len(probe) // 2], 1e-3))))
+            samples = sorted(_time_graph_replays(capture(graph_size), graph_size, max(warmup, 0), rep))
         return samples[len(samples) // 2]
 
     def add_measure(self, header: str, label: Any, fn: Callable[[], None], rep: int = 100) -> None:
