@@ -161,6 +161,19 @@ def test_every_plan_on_a_packed_weight_equals_the_row_major_result_bit_for_bit(m
     check_against_oracle(got, a, b, sa, sw, base=base)
 
 
+@pytest.mark.parametrize("m,n,k", [(7, 1000, 1024), (40, 2048, 4096), (64, 1040, 2048)])
+def test_float16_output_and_accumulation_on_a_packed_weight(m, n, k):
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=k + m, per_channel=True)
+    packed = _pack(b.t().view(torch.uint8))
+    base = torch.randn((m, n), device="cuda").to(torch.float16)
+    want, got = base.clone(), base.clone()
+    _run_fused(a, b, want, want, sa, sw, None, 0, None, None)    # base = D itself: accumulate in place
+    _run_fused(a, b, got, got, sa, sw, None, 0, None, packed)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    check_against_oracle(got, a, b, sa, sw, base=base)
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 1024, 1024), (8, 28672, 4096), (16, 2080, 2048), (5, 96, 256)])
 def test_swiglu_epilogue_on_a_packed_weight_equals_the_row_major_result(m, n, k):
     from hf_rocm_kernels import _capi
