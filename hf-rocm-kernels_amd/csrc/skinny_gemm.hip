@@ -40,11 +40,16 @@ __device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (
 
 // PACKED: the weight is in the pre-packed layout (pack_weight.hip), chunk (tile, kc) at (tile * k/256 + kc) * 4096 in
 // MFMA operand order: the loads are 1 KB contiguous per instruction and the chunk skips the transposition tile.
-template <int MT, int WN, int WK, int CH, bool PACKED>
+// RT = 16-row weight tiles per wave and chunk (1 or 2).  With 2 a wave's activation operands, read from LDS once per
+// 128 K-bytes, multiply two weight tiles: half the activation bytes through the LDS pipe per weight byte, which is what
+// bounds this kernel from 32 rows up.
+template <int MT, int WN, int WK, int CH, int RT, bool PACKED>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArgs a) {
     static_assert(WN * WK == kGemmWaves, "a workgroup is 8 waves");
+    static_assert(RT == 1 || RT == 2, "one or two weight tiles per wave");
     constexpr int KS = 256 * WK * CH;        // bytes of K per slab
-    constexpr int BN = 16 * WN;              // weight rows per panel
+    constexpr int BN = 16 * WN * RT;         // weight rows per panel
+    constexpr int ST = RT * MT;              // 16x16 output tiles per wave: index rt * MT + mt
     constexpr int ACT_BYTES = 16 * MT * KS;  // one staged activation slab
     constexpr int KP = KS / 16;              // 16-byte pieces per activation row of a slab
     constexpr int PIECES = 16 * MT * KP;
@@ -52,7 +57,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* const tbuf_all = lds;
-    uint8_t* const act_all = lds + kGemmWaves * kTileBytes;
+    uint8_t* const act_all = lds + kGemmWaves * RT * kTileBytes;
     int* const flag = reinterpret_cast<int*>(act_all + 2 * ACT_BYTES);
 
     const int tid = threadIdx.x;
@@ -77,9 +82,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // ---- per-panel epilogue inputs, fetched when the panel's first weight loads are issued -------------------
     // The vector-memory counter retires in issue order, so a load issued at the end of a panel would wait for
     // every prefetched weight chunk; issued up front, D and the channel scales are long home when needed.
-    // A lane owns D[mt*16 + li][n0 .. n0+3], n0 = panel*BN + wn*16 + 4*lg.  At most two panels are open at once.
-    uint2 dq[2][MT];
-    float sbq[2][4];
+    // A lane owns D[mt*16 + li][n0 .. n0+3], n0 = panel*BN + (wn*RT + rt)*16 + 4*lg.  At most two panels are open at once.
+    // With 8 output tiles per wave (64 rows x two weight tiles) there are no registers for that: the epilogue fetches.
+    constexpr bool kPrefetchEpilogue = ST < 8;
+    constexpr int kCtx = kPrefetchEpilogue ? 2 : 1;
+    uint2 dq[kCtx][ST];
+    float sbq[kCtx][RT][4];
     float saq[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -87,26 +95,29 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         saq[mt] = a.scale_a[(long)mrow * a.sa_stride];
     }
     const bool n_vec = (a.n & 3) == 0;
-    auto panel_fetch = [&](int panel, uint2 (&dd)[MT], float (&sb)[4]) __attribute__((always_inline)) {
-        const int n0 = panel * BN + wn * 16 + 4 * lg;
+    auto panel_fetch = [&](int panel, uint2 (&dd)[ST], float (&sb)[RT][4]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int n = min(n0 + v, a.n - 1);
-            sb[v] = a.scale_b ? a.scale_b[(long)n * a.sb_stride] : 1.0f;
-        }
+        for (int rt = 0; rt < RT; ++rt) {
+            const int n0 = panel * BN + (wn * RT + rt) * 16 + 4 * lg;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            dd[mt] = make_uint2(0u, 0u);
-            const int mrow = mt * 16 + li;
-            if (accumulate && mrow < a.m) {
-                const uint16_t* const drow = Dbase + (long)mrow * a.n;
-                if (n_vec && n0 + 3 < a.n) {
-                    dd[mt] = *reinterpret_cast<const uint2*>(drow + n0);
-                } else {
-                    uint32_t e[4];
+            for (int v = 0; v < 4; ++v) {
+                const int n = min(n0 + v, a.n - 1);
+                sb[rt][v] = a.scale_b ? a.scale_b[(long)n * a.sb_stride] : 1.0f;
+            }
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) e[v] = (n0 + v < a.n) ? drow[n0 + v] : 0u;
-                    dd[mt] = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+            for (int mt = 0; mt < MT; ++mt) {
+                dd[rt * MT + mt] = make_uint2(0u, 0u);
+                const int mrow = mt * 16 + li;
+                if (accumulate && mrow < a.m) {
+                    const uint16_t* const drow = Dbase + (long)mrow * a.n;
+                    if (n_vec && n0 + 3 < a.n) {
+                        dd[rt * MT + mt] = *reinterpret_cast<const uint2*>(drow + n0);
+                    } else {
+                        uint32_t e[4];
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) e[v] = (n0 + v < a.n) ? drow[n0 + v] : 0u;
+                        dd[rt * MT + mt] = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+                    }
                 }
             }
         }
@@ -116,7 +127,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // ---- weight stream -------------------------------------------------------------------------------------
     // load t of a chunk: lane -> weight row 4t + lane/16, bytes (lane%16)*16 .. +16 of the 256-byte chunk
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
-    v4i wq[2][CH][4];
+    v4i wq[2][CH][RT][4];
     int ip = u0 / S, is = u0 % S;  // (panel, slab) of the next unit to issue
     // Panel p walks its K slabs starting from slab p % S (sums do not care about the order): workgroups that move
     // through their panels in step then read different activation slabs at any moment instead of all hitting
@@ -132,29 +143,35 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // Weight chunk c of unit (ip, is) into register set X.
     auto issue_chunk = [&](auto sel, int c, bool in_range) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
-        if constexpr (PACKED) {
-            // a tile past the last one (n not a multiple of 16*WN) lies beyond the buffer and reads as zero
-            const uint32_t chunk = (uint32_t)(ip * WN + wn) * ((uint32_t)a.k >> 8) + (uint32_t)phys_slab(ip, is) * (WK * CH) + (uint32_t)(c * WK + wk);
-            const uint32_t base = in_range ? chunk * (uint32_t)kTileBytes + (uint32_t)lane * 16u : 0x80000000u;
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(base + (uint32_t)t * 1024u), 0, 2 /* nt */);
-        } else {
-            const uint32_t base = in_range ? (uint32_t)(ip * BN + wn * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
-                                                 (uint32_t)(c * WK + wk) * 256u
-                                           : 0x80000000u;
+        for (int rt = 0; rt < RT; ++rt) {
+            const int tile = ip * (WN * RT) + wn * RT + rt;  // 16-row weight tile
+            if constexpr (PACKED) {
+                // a tile past the last one (n not a multiple of the panel height) lies beyond the buffer and reads as zero
+                const uint32_t chunk = (uint32_t)tile * ((uint32_t)a.k >> 8) + (uint32_t)phys_slab(ip, is) * (WK * CH) + (uint32_t)(c * WK + wk);
+                const uint32_t base = in_range ? chunk * (uint32_t)kTileBytes + (uint32_t)lane * 16u : 0x80000000u;
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                wq[X][c][t] = __builtin_amdgcn_raw_buffer_load_b128(
-                    w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+                for (int t = 0; t < 4; ++t)
+                    wq[X][c][rt][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(base + (uint32_t)t * 1024u), 0, 2 /* nt */);
+            } else {
+                const uint32_t base = in_range ? (uint32_t)(tile * 16) * (uint32_t)a.b_stride + (uint32_t)phys_slab(ip, is) * KS +
+                                                     (uint32_t)(c * WK + wk) * 256u
+                                               : 0x80000000u;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    wq[X][c][rt][t] = __builtin_amdgcn_raw_buffer_load_b128(
+                        w_rsrc, (int)(w_lane_off + base + (uint32_t)(4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+            }
         }
     };
     // Epilogue inputs of unit (ip, is) if it opens a panel, then move on to the next unit.
     auto issue_done = [&](bool in_range) __attribute__((always_inline)) {
         if (in_range && issue_first) {
-            if (wk == 0) {
-                if (fetch_par) panel_fetch(ip, dq[1], sbq[1]);
-                else panel_fetch(ip, dq[0], sbq[0]);
+            if constexpr (kPrefetchEpilogue) {
+                if (wk == 0) {
+                    if (fetch_par) panel_fetch(ip, dq[kCtx - 1], sbq[kCtx - 1]);
+                    else panel_fetch(ip, dq[0], sbq[0]);
+                }
             }
             fetch_par ^= 1;
         }
@@ -194,11 +211,11 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         }
     };
 
-    v4f acc[MT];
+    v4f acc[ST];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int st = 0; st < ST; ++st) acc[st] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    uint8_t* const tb = tbuf_all + wave * kTileBytes;
+    uint8_t* const tb = tbuf_all + wave * RT * kTileBytes;  // this wave's RT transposition tiles
     // swizzled offsets of this lane inside a 16 x 256 B tile: as writer (row 4t+lg, piece li) and as reader (row li)
     int wr_off[4];
 #pragma unroll
@@ -217,12 +234,14 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         const uint8_t* const act = act_all + buf * ACT_BYTES;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            v4i wcur[4];  // PACKED: the chunk's operands, out of the way of the next request
+            v4i wcur[RT][4];  // PACKED: the chunk's operands, out of the way of the next request
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                if constexpr (PACKED) wcur[t] = wq[X][c][t];
-                else *reinterpret_cast<v4i*>(tb + wr_off[t]) = wq[X][c][t];
-            }
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    if constexpr (PACKED) wcur[rt][t] = wq[X][c][rt][t];
+                    else *reinterpret_cast<v4i*>(tb + rt * kTileBytes + wr_off[t]) = wq[X][c][rt][t];
+                }
             issue_chunk(sel, c, next_in_range);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -230,22 +249,28 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             const int kblk = c * WK + wk;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                v4i wlo, whi;
-                if constexpr (PACKED) {
-                    wlo = wcur[2 * h];
-                    whi = wcur[2 * h + 1];
-                } else {
-                    wlo = *reinterpret_cast<const v4i*>(tb + li * 256 + rd_off[h]);
-                    whi = *reinterpret_cast<const v4i*>(tb + li * 256 + (rd_off[h] ^ 16));
+                v8i wop[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    v4i wlo, whi;
+                    if constexpr (PACKED) {
+                        wlo = wcur[rt][2 * h];
+                        whi = wcur[rt][2 * h + 1];
+                    } else {
+                        wlo = *reinterpret_cast<const v4i*>(tb + rt * kTileBytes + li * 256 + rd_off[h]);
+                        whi = *reinterpret_cast<const v4i*>(tb + rt * kTileBytes + li * 256 + (rd_off[h] ^ 16));
+                    }
+                    wop[rt] = v8i{wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
                 }
-                const v8i wop = {wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     const uint8_t* const arow = act + (mt * 16 + li) * KS + kblk * 256;
                     const v4i alo = *reinterpret_cast<const v4i*>(arow + rd_off[h]);
                     const v4i ahi = *reinterpret_cast<const v4i*>(arow + (rd_off[h] ^ 16));
                     const v8i aop = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
-                    acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, aop, acc[mt], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        acc[rt * MT + mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[rt], aop, acc[rt * MT + mt], 0, 0, 0, 0, 0, 0);
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -256,18 +281,23 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // ---- epilogue ------------------------------------------------------------------------------------------
     // lane holds, per m-tile, D^T[n0 + v][mt*16 + li], v = 0..3: scale, add the fetched D, round once, store
     auto store_panel = [&](int panel, int par) __attribute__((always_inline)) {
-        const int n0 = panel * BN + wn * 16 + 4 * lg;
-        const bool vec_ok = n_vec && (n0 + 3 < a.n);
+        if constexpr (!kPrefetchEpilogue) {
+            panel_fetch(panel, dq[0], sbq[0]);
+            par = 0;
+        }
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
+        for (int st = 0; st < ST; ++st) {
+            const int rt = st / MT, mt = st % MT;
+            const int n0 = panel * BN + (wn * RT + rt) * 16 + 4 * lg;
+            const bool vec_ok = n_vec && (n0 + 3 < a.n);
             const int mrow = mt * 16 + li;
             if (mrow >= a.m) continue;
-            const uint2 old = par ? dq[1][mt] : dq[0][mt];
+            const uint2 old = par ? dq[kCtx - 1][st] : dq[0][st];
             const uint32_t oe[4] = {old.x & 0xffffu, old.x >> 16, old.y & 0xffffu, old.y >> 16};
             uint32_t o[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const float r = acc[mt][v] * (saq[mt] * (par ? sbq[1][v] : sbq[0][v]));
+                const float r = acc[st][v] * (saq[mt] * (par ? sbq[kCtx - 1][rt][v] : sbq[0][rt][v]));
                 const float base = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>((uint16_t)oe[v]) : load16<HFRK_F16>((uint16_t)oe[v]);
                 const float sum = accumulate ? base + r : r;
                 o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
@@ -283,12 +313,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         }
     };
 
-    // fp32 partial of (workgroup gg, slot): [wn][mt][lane] float4.  Partials cross XCDs, whose L2s are not coherent
+    // fp32 partial of (workgroup gg, slot): [wn][rt * MT + mt][lane] float4.  Partials cross XCDs, whose L2s are not coherent
     // with each other: they are written through to memory and read past the caches (sc0 sc1 on both sides), which
     // keeps them coherent per location without the L2 write-back / invalidate a device-scope fence would cost.
     const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
-    auto ws_off = [&](int gg, int slot, int mt) __attribute__((always_inline)) -> int {
-        return (((gg * 2 + slot) * (WN * MT) + wn * MT + mt) * 64 + lane) * 16;
+    auto ws_off = [&](int gg, int slot, int st) __attribute__((always_inline)) -> int {
+        return (((gg * 2 + slot) * (WN * ST) + wn * ST + st) * 64 + lane) * 16;
     };
     constexpr int kCoherent = 17;  // sc0 | sc1
 
@@ -300,15 +330,15 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             v4f* const mine = reinterpret_cast<v4f*>(tb);
             if (wk != 0) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) mine[mt * 64 + lane] = acc[mt];
+                for (int st = 0; st < ST; ++st) mine[st * 64 + lane] = acc[st];
             }
             __syncthreads();
             if (wk == 0) {
 #pragma unroll
                 for (int w = 1; w < WK; ++w) {
-                    const v4f* const other = reinterpret_cast<const v4f*>(tbuf_all + (wn * WK + w) * kTileBytes);
+                    const v4f* const other = reinterpret_cast<const v4f*>(tbuf_all + (wn * WK + w) * RT * kTileBytes);
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) acc[mt] += other[mt * 64 + lane];
+                    for (int st = 0; st < ST; ++st) acc[st] += other[st * 64 + lane];
                 }
             }
             __syncthreads();
@@ -320,8 +350,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             const int slot = (panel == u0 / S) ? 0 : 1;
             if (wk == 0) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, acc[mt]), ws_rsrc, ws_off(g, slot, mt), 0, kCoherent);
+                for (int st = 0; st < ST; ++st)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, acc[st]), ws_rsrc, ws_off(g, slot, st), 0, kCoherent);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stores acknowledged before the arrival is counted
             }
             __syncthreads();
@@ -340,12 +370,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                 const int g_first = (int)(((lo + 1) * (uint32_t)G + (uint32_t)U - 1) / (uint32_t)U) - 1;
                 const int g_last = (int)((hi * (uint32_t)G + (uint32_t)U - 1) / (uint32_t)U) - 1;
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+                for (int st = 0; st < ST; ++st) acc[st] = v4f{0.f, 0.f, 0.f, 0.f};
                 for (int gg = g_first; gg <= g_last; ++gg) {
                     const int sl = (unit_begin(gg, U, G) / S == panel) ? 0 : 1;
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[mt] += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_off(gg, sl, mt), 0, kCoherent));
+                    for (int st = 0; st < ST; ++st)
+                        acc[st] += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_off(gg, sl, st), 0, kCoherent));
                 }
                 store_panel(panel, flush_par);
             }
@@ -353,7 +383,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         }
         flush_par ^= 1;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int st = 0; st < ST; ++st) acc[st] = v4f{0.f, 0.f, 0.f, 0.f};
     };
 
     // ---- main loop -----------------------------------------------------------------------------------------
@@ -438,8 +468,8 @@ static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
     return HFRK_SUCCESS;
 }
 
-constexpr int lds_bytes_for(int mt, int wk, int ch) {
-    return kGemmWaves * kTileBytes + 2 * 16 * mt * (256 * wk * ch) + 16;
+constexpr int lds_bytes_for(int mt, int wk, int ch, int rt = 1) {
+    return kGemmWaves * rt * kTileBytes + 2 * 16 * mt * (256 * wk * ch) + 16;
 }
 
 // m <= 32: every wave streams its own run of (16*RT-row group, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
@@ -585,21 +615,25 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p)
         return HFRK_SUCCESS;
     }
     if (p->m_tiles < 1 || p->m_tiles > 4 || p->m_tiles * 16 < m) return HFRK_INVALID_CONFIG;
-    if (!(p->wn == 1 || p->wn == 2 || p->wn == 4 || p->wn == 8) || p->wn * p->wk != kGemmWaves) return HFRK_INVALID_CONFIG;
+    // wn counts the 16-row tiles of a panel: one per row wave (wn * wk = 8) or, with one chunk per slab, two (wn * wk = 16)
+    if (!(p->wk == 1 || p->wk == 2 || p->wk == 4 || p->wk == 8)) return HFRK_INVALID_CONFIG;
+    const int rt = p->wn * p->wk / kGemmWaves;
+    if (p->wn < 1 || p->wn * p->wk != rt * kGemmWaves || (rt != 1 && rt != 2)) return HFRK_INVALID_CONFIG;
     if (p->ch != 1 && p->ch != 2) return HFRK_INVALID_CONFIG;
+    if (rt == 2 && (p->ch != 1 || p->grid > kMaxGrid / 2)) return HFRK_INVALID_CONFIG;  // registers; workspace slots are twice as large
     const int ks = 256 * p->wk * p->ch, bn = 16 * p->wn;
     if (k % ks != 0 || p->slabs != k / ks || p->panels != (n + bn - 1) / bn) return HFRK_INVALID_CONFIG;
     if (p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
     const long units = (long)p->panels * p->slabs;
     if (p->grid < 1 || p->grid > kMaxGrid || p->grid > units) return HFRK_INVALID_CONFIG;
     if (units * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's unit arithmetic is 32-bit
-    if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
+    if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch, rt) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
     return HFRK_SUCCESS;
 }
 
-template <int MT, int WN, int WK, int CH, bool PACKED>
+template <int MT, int WN, int WK, int CH, int RT, bool PACKED>
 static int launch_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_kernel<MT, WN, WK, CH, PACKED>;
+    auto kern = skinny_gemm_kernel<MT, WN, WK, CH, RT, PACKED>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -612,21 +646,23 @@ static int launch_packing(const GemmArgs& args, int lds_bytes, hipStream_t strea
     return HFRK_SUCCESS;
 }
 
-template <int MT, int WN, int WK, int CH>
+template <int MT, int WN, int WK, int CH, int RT>
 static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    return args.packed ? launch_packing<MT, WN, WK, CH, true>(args, lds_bytes, stream)
-                       : launch_packing<MT, WN, WK, CH, false>(args, lds_bytes, stream);
+    return args.packed ? launch_packing<MT, WN, WK, CH, RT, true>(args, lds_bytes, stream)
+                       : launch_packing<MT, WN, WK, CH, RT, false>(args, lds_bytes, stream);
 }
 
 template <int MT>
 static int launch_mt(const GemmArgs& args, const hfrk_gemm_plan& p, hipStream_t stream) {
     // decompositions whose activation slabs cannot fit in LDS are never planned and are not compiled
-#define HFRK_CASE(WN_, WK_, CH_)                                                             \
-    if constexpr (lds_bytes_for(MT, WK_, CH_) <= kLdsLimit) {                                \
-        if (p.wn == WN_ && p.ch == CH_) return launch_one<MT, WN_, WK_, CH_>(args, p.lds_bytes, stream); \
+    // WN_ = row waves; the plan's wn = WN_ * RT_ tiles per panel
+#define HFRK_CASE(WN_, WK_, CH_, RT_)                                                        \
+    if constexpr (lds_bytes_for(MT, WK_, CH_, RT_) <= kLdsLimit) {                           \
+        if (p.wn == WN_ * RT_ && p.wk == WK_ && p.ch == CH_) return launch_one<MT, WN_, WK_, CH_, RT_>(args, p.lds_bytes, stream); \
     }
-    HFRK_CASE(1, 8, 1) HFRK_CASE(1, 8, 2) HFRK_CASE(2, 4, 1) HFRK_CASE(2, 4, 2)
-    HFRK_CASE(4, 2, 1) HFRK_CASE(4, 2, 2) HFRK_CASE(8, 1, 1) HFRK_CASE(8, 1, 2)
+    HFRK_CASE(1, 8, 1, 1) HFRK_CASE(1, 8, 2, 1) HFRK_CASE(2, 4, 1, 1) HFRK_CASE(2, 4, 2, 1)
+    HFRK_CASE(4, 2, 1, 1) HFRK_CASE(4, 2, 2, 1) HFRK_CASE(8, 1, 1, 1) HFRK_CASE(8, 1, 2, 1)
+    HFRK_CASE(1, 8, 1, 2) HFRK_CASE(2, 4, 1, 2) HFRK_CASE(4, 2, 1, 2) HFRK_CASE(8, 1, 1, 2)
 #undef HFRK_CASE
     return HFRK_INVALID_CONFIG;
 }

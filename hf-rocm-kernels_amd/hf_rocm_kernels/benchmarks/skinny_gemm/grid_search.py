@@ -44,15 +44,15 @@ def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.Gemm
             for g in grids:
                 plans.append(_capi.GemmPlan(mt, -1, wave_k // 256, 0, min(g, 256, tiles * windows), tiles, windows,
                                             8 * (wave_k // 256) * 4096 + 16 * mt * 1024))
-    for wn, ch in itertools.product((1, 2, 4, 8), (1, 2)):  # workgroup
+    for wn, ch, rt in itertools.product((1, 2, 4, 8), (1, 2), (1, 2)):  # workgroup: row waves, chunks per slab, tiles per wave
         wk = 8 // wn
         ks = 256 * wk * ch
-        lds = 8 * 4096 + 2 * 16 * mt * ks + 16
-        if k % ks or lds > 160 * 1024:
+        lds = 8 * rt * 4096 + 2 * 16 * mt * ks + 16
+        if k % ks or lds > 160 * 1024 or (rt == 2 and ch != 1):
             continue
-        panels, slabs = -(-n // (16 * wn)), k // ks
+        panels, slabs = -(-n // (16 * wn * rt)), k // ks
         for g in grids:
-            plans.append(_capi.GemmPlan(mt, wn, wk, ch, min(g, panels * slabs), panels, slabs, lds))
+            plans.append(_capi.GemmPlan(mt, wn * rt, wk, ch, min(g, panels * slabs, 512 if rt == 2 else 1024), panels, slabs, lds))
     return plans
 
 
@@ -61,7 +61,8 @@ def describe(p: _capi.GemmPlan) -> str:
         return f"wave-stream row_tiles={p.wk} act_loads={p.ch} grid={p.grid}"
     if p.wn == -1:
         return f"k-split wave_k={256 * p.wk} windows={p.slabs} grid={p.grid}"
-    return f"workgroup wn={p.wn} wk={p.wk} ch={p.ch} grid={p.grid}"
+    tiles_per_wave = p.wn * p.wk // 8
+    return f"workgroup wn={p.wn // tiles_per_wave} wk={p.wk} ch={p.ch} rt={tiles_per_wave} grid={p.grid}"
 
 
 def time_plan(lib, arena: torch.Tensor, m: int, n: int, k: int, plan, reps: int, packed: bool = False) -> float:

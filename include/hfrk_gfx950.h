@@ -58,8 +58,9 @@ typedef struct hfrk_gemm_plan {
     int wn;        /* which decomposition:
                        0          wave-stream (m <= 32): every wave streams its own run of chunks
                       -1          K-split (k % (2048*wk) == 0): the 8 waves of a workgroup split K, activations in registers
-                       1,2,4,8    workgroup: wn waves spread over output rows (16 weight rows each), wk over K */
-    int wk;        /* workgroup: waves spread over K, wn*wk = 8.  wave-stream: 16-row weight tiles per chunk (1 or 2).
+                       1..16      workgroup: a panel is wn 16-row weight tiles; the 8 waves are 8/wk row waves x wk K waves,
+                                  each row wave takes wn*wk/8 tiles (1, or 2 with ch = 1) */
+    int wk;        /* workgroup: waves spread over K (1, 2, 4, 8), wn*wk = 8 or 16.  wave-stream: 16-row weight tiles per chunk (1 or 2).
                       K-split: bytes of K per wave / 256 (1, 2, or 4 with m_tiles <= 2) */
     int ch;        /* workgroup: 256-byte K chunks each wave streams per slab (1 or 2).
                       wave-stream: 16-byte activation loads per lane and chunk, ceil(m/4).  K-split: 0 */

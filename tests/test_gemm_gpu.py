@@ -70,20 +70,20 @@ def all_plans(m, n, k):
             tiles, windows = (n + 15) // 16, k // (8 * wave_k)
             for grid in sorted({min(g, tiles * windows) for g in (256, 200, 7, 1)}):
                 plans.append(_capi.GemmPlan(mt, -1, wave_k // 256, 0, grid, tiles, windows, 8 * (wave_k // 256) * 4096 + 16 * mt * 1024))
-    for wn in (1, 2, 4, 8):
+    for wn, rt in [(w, r) for w in (1, 2, 4, 8) for r in (1, 2)]:  # row waves x weight tiles per wave
         wk = 8 // wn
-        for ch in (1, 2):
+        for ch in ((1, 2) if rt == 1 else (1,)):
             ks = 256 * wk * ch
             if k % ks:
                 continue
-            lds = 8 * 4096 + 2 * 16 * mt * ks + 16
+            lds = 8 * rt * 4096 + 2 * 16 * mt * ks + 16
             if lds > 160 * 1024:
                 continue
-            panels = (n + 16 * wn - 1) // (16 * wn)
+            panels = (n + 16 * wn * rt - 1) // (16 * wn * rt)
             slabs = k // ks
             units = panels * slabs
             for grid in sorted({min(256, units), min(200, units), min(7, units)}):
-                p = _capi.GemmPlan(mt, wn, wk, ch, grid, panels, slabs, lds)
+                p = _capi.GemmPlan(mt, wn * rt, wk, ch, grid, panels, slabs, lds)
                 plans.append(p)
     return plans
 
