@@ -280,18 +280,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 
     // ---- epilogue ------------------------------------------------------------------------------------------
     // lane holds, per m-tile, D^T[n0 + v][mt*16 + li], v = 0..3: scale, add the fetched D, round once, store
-    // Called by every wave of the workgroup; `active` marks the waves that hold the finished sums (wk == 0).
-    // From 17 rows up, and when the panel's columns are whole 16-byte pieces of D's rows, the 16-bit results go through
-    // LDS (the transposition tiles are idle here) and leave as whole row segments, 4 rows x 2*BN contiguous bytes per
-    // store instruction; written from the accumulator layout every instruction would touch 32-byte pieces of 16
-    // different rows, which at 64 rows takes three times as long as the stores of a 16-row result.
-    constexpr int kRowPitch = BN * 2 + 16;  // bytes per staged row; the pad spreads the rows over the LDS banks
-    static_assert(16 * MT * kRowPitch <= kGemmWaves * RT * kTileBytes, "the staged panel fits the transposition tiles");
-    const bool stage_rows = MT >= 2 && (a.n & 7) == 0 && (reinterpret_cast<uintptr_t>(a.D) & 15) == 0;
-    auto store_panel = [&](int panel, int par, bool active) __attribute__((always_inline)) {
-        const bool staged = stage_rows && (panel * BN + BN <= a.n);  // uniform over the workgroup
-        if (!staged && !active) return;
-        if (active) {
+    auto store_panel = [&](int panel, int par) __attribute__((always_inline)) {
         if constexpr (!kPrefetchEpilogue) {
             panel_fetch(panel, dq[0], sbq[0]);
             par = 0;
@@ -302,7 +291,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             const int n0 = panel * BN + (wn * RT + rt) * 16 + 4 * lg;
             const bool vec_ok = n_vec && (n0 + 3 < a.n);
             const int mrow = mt * 16 + li;
-            if (mrow >= a.m && !staged) continue;
+            if (mrow >= a.m) continue;
             const uint2 old = par ? dq[kCtx - 1][st] : dq[0][st];
             const uint32_t oe[4] = {old.x & 0xffffu, old.x >> 16, old.y & 0xffffu, old.y >> 16};
             uint32_t o[4];
@@ -313,11 +302,6 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                 const float sum = accumulate ? base + r : r;
                 o[v] = a.d_dtype == HFRK_BF16 ? store16<HFRK_BF16>(sum) : store16<HFRK_F16>(sum);
             }
-            if (staged) {  // rows >= m are staged too and dropped below
-                *reinterpret_cast<uint2*>(tbuf_all + mrow * kRowPitch + ((wn * RT + rt) * 16 + 4 * lg) * 2) =
-                    make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
-                continue;
-            }
             uint16_t* const drow = D + (long)mrow * a.n;
             if (vec_ok) {
                 *reinterpret_cast<uint2*>(drow + n0) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
@@ -326,19 +310,6 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                 for (int v = 0; v < 4; ++v)
                     if (n0 + v < a.n) drow[n0 + v] = (uint16_t)o[v];
             }
-        }
-        }
-        if (staged) {
-            __syncthreads();
-            constexpr int kPiecesPerRow = BN / 8;  // 16-byte pieces of a row segment
-#pragma unroll 1
-            for (int p = tid; p < 16 * MT * kPiecesPerRow; p += kGemmThreads) {
-                const int row = p / kPiecesPerRow, piece = p % kPiecesPerRow;
-                if (row < a.m)
-                    *reinterpret_cast<v4i*>(D + (long)row * a.n + panel * BN + piece * 8) =
-                        *reinterpret_cast<const v4i*>(tbuf_all + row * kRowPitch + piece * 16);
-            }
-            __syncthreads();  // the tiles are written again by the next unit
         }
     };
 
@@ -374,7 +345,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
         }
         const bool full = (s_first == 0) && (s_end == S);
         if (full) {
-            store_panel(panel, flush_par, wk == 0);
+            if (wk == 0) store_panel(panel, flush_par);
         } else {
             const int slot = (panel == u0 / S) ? 0 : 1;
             if (wk == 0) {
@@ -406,8 +377,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                     for (int st = 0; st < ST; ++st)
                         acc[st] += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_off(gg, sl, st), 0, kCoherent));
                 }
+                store_panel(panel, flush_par);
             }
-            if (last) store_panel(panel, flush_par, wk == 0);  // `last` is uniform: every wave takes part in the staged store
             __syncthreads();  // `flag` may be rewritten by the next flush
         }
         flush_par ^= 1;
