@@ -255,9 +255,15 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             const int kblk = c * WK + wk;
+            // Every operand of the chunk is requested from LDS before the first MFMA: one LDS latency per chunk instead
+            // of one per pair of MFMAs (the LDS answers in order, so the MFMAs start as their operands arrive).  The
+            // variants with the most accumulators and prefetch registers do it per 128-byte K step: two latencies.
+            constexpr int HB = (MT >= 3 && (CH == 2 || RT == 2)) ? 1 : 2;  // K steps requested together
+            v8i wop[2][RT], aop[2][MT];
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                v8i wop[RT];
+            for (int h0 = 0; h0 < 2; h0 += HB) {
+#pragma unroll
+            for (int h = h0; h < h0 + HB; ++h) {
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
                     v4i wlo, whi;
@@ -268,18 +274,24 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                         wlo = *reinterpret_cast<const v4i*>(tb + rt * kTileBytes + li * 256 + rd_off[h]);
                         whi = *reinterpret_cast<const v4i*>(tb + rt * kTileBytes + li * 256 + (rd_off[h] ^ 16));
                     }
-                    wop[rt] = v8i{wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
+                    wop[h][rt] = v8i{wlo[0], wlo[1], wlo[2], wlo[3], whi[0], whi[1], whi[2], whi[3]};
                 }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     const uint8_t* const arow = act + (mt * 16 + li) * KS + kblk * 256;
                     const v4i alo = *reinterpret_cast<const v4i*>(arow + rd_off[h]);
                     const v4i ahi = *reinterpret_cast<const v4i*>(arow + (rd_off[h] ^ 16));
-                    const v8i aop = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+                    aop[h][mt] = v8i{alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests above ahead of the MFMAs below
+#pragma unroll
+            for (int h = h0; h < h0 + HB; ++h)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
-                        acc[rt * MT + mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[rt], aop, acc[rt * MT + mt], 0, 0, 0, 0, 0, 0);
-                }
+                        acc[rt * MT + mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h][rt], aop[h][mt], acc[rt * MT + mt], 0, 0, 0, 0, 0, 0);
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();

@@ -206,6 +206,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
         for (int mt = 0; mt < MT; ++mt) acc[mt] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KCH; ++c) {
+            // both weight operands of the column chunk are requested from LDS before its first MFMA
+            v8i wop[2];
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 v4i lo, hi;
@@ -216,11 +218,13 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
                     lo = *reinterpret_cast<const v4i*>(tw + c * kTileBytes + rd_off[h]);
                     hi = *reinterpret_cast<const v4i*>(tw + c * kTileBytes + (rd_off[h] ^ 16));
                 }
-                const v8i wop = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                wop[h] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
-                    acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop, areg[mt][2 * c + h], acc[mt], 0, 0, 0, 0, 0, 0);
-            }
+                    acc[mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h], areg[mt][2 * c + h], acc[mt], 0, 0, 0, 0, 0, 0);
             if constexpr (PACKED) {
                 if (more) issue_chunk(c, 0u);
             }

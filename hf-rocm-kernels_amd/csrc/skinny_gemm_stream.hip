@@ -268,9 +268,11 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // every operand of the chunk is requested from LDS before the first MFMA: one LDS latency per chunk, and the
+        // MFMAs start as their operands arrive (the LDS answers in order)
+        v8i wop[2][RT], aop[2][MT];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            v8i wop[RT], aop[MT];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 v4i lo, hi;
@@ -281,20 +283,23 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
                     lo = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + rd_off[h]);
                     hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
                 }
-                wop[rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                wop[h][rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const v4i lo = *reinterpret_cast<const v4i*>(ta + mt * kTileBytes + rd_off[h]);
                 const v4i hi = *reinterpret_cast<const v4i*>(ta + mt * kTileBytes + (rd_off[h] ^ 16));
-                aop[mt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                aop[h][mt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests above ahead of the MFMAs below
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
-                    acc[rt * MT + mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[rt], aop[mt], acc[rt * MT + mt], 0, 0, 0, 0, 0, 0);
-        }
+                    acc[rt * MT + mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h][rt], aop[h][mt], acc[rt * MT + mt], 0, 0, 0, 0, 0, 0);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if (++kc == KC) {  // a row tile ends inside this wave's run
