@@ -48,8 +48,8 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
 
 HBM_PEAK_GBPS = 8000.0
 # Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0099 x the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55240479}
+# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0097 x the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55228662}
 CALIBRATION_COPY_BYTES = 256 << 20
 
 WORKLOADS = {
@@ -60,7 +60,7 @@ WORKLOADS = {
                 "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-8B decode shapes, M=1..16 (us/call in `cases`)",
         "kernel": "hfrk::skinny_gemm_stream_kernel (16 of the 20 launches of a step); with the shipped plan table "
-                  "hfrk::skinny_gemm_kernel<1,8,1,2> on gate_up at M=1,8,16 and hfrk::skinny_gemm_ksplit_kernel<1,512> on qkv at M=16",
+                  "hfrk::skinny_gemm_kernel<1,8,1,2,1,2> on gate_up at M=8,16 and hfrk::skinny_gemm_ksplit_kernel<1,512> on qkv at M=16",
     },
     "llama3-70b": {
         "shapes": [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)],
