@@ -365,3 +365,26 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
     plan_table.clear()
     assert plan_table.load(str(other), strict=False) == 1
     plan_table.clear()
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (16, 28672, 4096), (32, 4096, 14336), (64, 8192, 8192),
+                                   (40, 1000, 2048), (17, 50, 256)])
+def test_every_plan_the_sweep_tool_proposes_is_one_the_library_accepts(m, n, k):
+    """benchmarks/skinny_gemm/grid_search.py enumerates hfrk_gemm_plan structs by its own arithmetic; the library
+    validates plans with its own (hfrk_plan_table_set runs the launcher's check, no device needed).  They must agree,
+    for every decomposition family, and describe() must name each one."""
+    from hf_rocm_kernels import plan_table
+    from hf_rocm_kernels.benchmarks.skinny_gemm import grid_search
+    plans = grid_search.candidate_plans(m, n, k, [7, 160, 224, 256, 512])
+    assert plans
+    families = set()
+    plan_table.clear()
+    try:
+        for p in plans:
+            status = _capi.load().hfrk_plan_table_set(m, n, k, 0, ctypes.byref(p))
+            assert status == _capi.SUCCESS, (grid_search.describe(p), p.as_dict(), _capi.status_string(status))
+            families.add(grid_search.describe(p).split()[0])
+    finally:
+        plan_table.clear()
+    assert "workgroup" in families
+    assert ("wave-stream" in families) == (m <= 32)
