@@ -43,16 +43,10 @@ __device__ __forceinline__ int unit_begin(int g, int units, int grid) { return (
 // RT = 16-row weight tiles per wave and chunk (1 or 2).  With 2 a wave's activation operands, read from LDS once per
 // 128 K-bytes, multiply two weight tiles: half the activation bytes through the LDS pipe per weight byte, which is what
 // bounds this kernel from 32 rows up.
-// NBUF = staged activation slabs in LDS.  With 2 a barrier per unit hands the next slab over, which keeps the 8 waves in
-// lockstep: they queue on the LDS pipe together and then wait for memory together.  With 3 the hand-over is two
-// counters per slab in LDS ("all waves have stored their part", "all waves are done reading it"), a wave only waits
-// when it is a whole unit ahead of the slowest one, and the LDS phase of one wave overlaps the memory wait of another.
-// Every wait is bounded: if a counter never arrives the wave goes on (the result is then wrong, the kernel still ends).
-template <int MT, int WN, int WK, int CH, int RT, int NBUF, bool PACKED>
+template <int MT, int WN, int WK, int CH, int RT, bool PACKED>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArgs a) {
     static_assert(WN * WK == kGemmWaves, "a workgroup is 8 waves");
     static_assert(RT == 1 || RT == 2, "one or two weight tiles per wave");
-    static_assert(NBUF == 2 || NBUF == 3, "two or three activation slabs");
     constexpr int KS = 256 * WK * CH;        // bytes of K per slab
     constexpr int BN = 16 * WN * RT;         // weight rows per panel
     constexpr int ST = RT * MT;              // 16x16 output tiles per wave: index rt * MT + mt
@@ -64,9 +58,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* const tbuf_all = lds;
     uint8_t* const act_all = lds + kGemmWaves * RT * kTileBytes;
-    int* const flag = reinterpret_cast<int*>(act_all + NBUF * ACT_BYTES);
-    int* const stored = flag + 4;    // NBUF == 3: waves that have stored their part of the slab in buffer b, ever
-    int* const consumed = flag + 8;  //            waves that have finished reading buffer b, ever
+    int* const flag = reinterpret_cast<int*>(act_all + 2 * ACT_BYTES);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -415,63 +407,26 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     int s_first = cs;              // first slab this workgroup covers of the current panel
     auto next_slab = [&](int s) __attribute__((always_inline)) { return (s + 1 == S) ? 0 : s + 1; };
 
-    constexpr int kSpinLimit = 1 << 20;
-    auto signal = [&](int* counter) __attribute__((always_inline)) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this wave's LDS accesses so far are done
-        if (lane == 0) __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    };
-    auto wait_for = [&](int* counter, int target) __attribute__((always_inline)) {
-        int spins = 0;
-        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target && ++spins < kSpinLimit)
-            __builtin_amdgcn_s_sleep(1);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    };
-    if constexpr (NBUF == 3) {
-        if (tid < 3) stored[tid] = 0;
-        else if (tid < 6) consumed[tid - 3] = 0;
-        __syncthreads();
-    }
-
     act_load(true);
     issue_unit(Sel0{}, true);
     act_store(0);
-    if constexpr (NBUF == 3) signal(&stored[0]);
     act_load(u0 + 1 < u1);
     issue_unit(Sel1{}, u0 + 1 < u1);
-    if constexpr (NBUF == 2) __syncthreads();
-    int bcur = 0, fill = 0;  // NBUF == 3: buffer of the unit being consumed (unit index % 3) and how often it was filled before
+    __syncthreads();
 
     // One step = one unit.  A step whose unit lies past u1 (odd range length) multiplies zeros and changes nothing.
     auto step = [&](auto sel, int u) __attribute__((always_inline)) {
         constexpr int X = decltype(sel)::value;
         const int ns = next_slab(cs);
-        if constexpr (NBUF == 2) {
-            if (u + 1 < u1) act_store(X ^ 1);  // slab of unit u+1, requested one step ago
-            act_load(u + 2 < u1);
-            consume_unit(sel, X, u + 2 < u1);
-        } else {
-            const int bnext = bcur == 2 ? 0 : bcur + 1;     // buffer of unit u+1
-            const int fill_next = bcur == 2 ? fill + 1 : fill;  // fills of that buffer before this one
-            if (u + 1 < u1) {
-                wait_for(&consumed[bnext], kGemmWaves * fill_next);  // its previous slab (unit u-2) has been read by all
-                act_store(bnext);
-                signal(&stored[bnext]);
-            }
-            act_load(u + 2 < u1);
-            if (u < u1) wait_for(&stored[bcur], kGemmWaves * (fill + 1));  // every wave's part of this unit's slab is there
-            consume_unit(sel, bcur, u + 2 < u1);
-            if (u < u1) signal(&consumed[bcur]);
-            bcur = bnext;
-            fill = fill_next;
-        }
+        if (u + 1 < u1) act_store(X ^ 1);  // slab of unit u+1, requested one step ago
+        act_load(u + 2 < u1);
+        consume_unit(sel, X, u + 2 < u1);
         if (u < u1 && (u + 1 == u1 || ns == 0)) {
             flush_panel(cp, s_first, cs + 1);
             s_first = 0;
         }
         issue_done(u + 2 < u1);
-        if constexpr (NBUF == 2) {
-            if (u + 1 < u1) __syncthreads();
-        }
+        if (u + 1 < u1) __syncthreads();
         cs = ns;
         if (ns == 0) ++cp;
     };
@@ -525,8 +480,8 @@ static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
     return HFRK_SUCCESS;
 }
 
-constexpr int lds_bytes_for(int mt, int wk, int ch, int rt = 1, int nbuf = 2) {
-    return kGemmWaves * rt * kTileBytes + nbuf * 16 * mt * (256 * wk * ch) + (nbuf == 3 ? 64 : 16);
+constexpr int lds_bytes_for(int mt, int wk, int ch, int rt = 1) {
+    return kGemmWaves * rt * kTileBytes + 2 * 16 * mt * (256 * wk * ch) + 16;
 }
 
 // m <= 32: every wave streams its own run of (16*RT-row group, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
@@ -684,15 +639,13 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p)
     const long units = (long)p->panels * p->slabs;
     if (p->grid < 1 || p->grid > kMaxGrid || p->grid > units) return HFRK_INVALID_CONFIG;
     if (units * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's unit arithmetic is 32-bit
-    // two staged activation slabs, or (from 17 rows) three: the plan says which through its LDS size
-    const bool three = p->m_tiles >= 2 && p->lds_bytes == lds_bytes_for(p->m_tiles, p->wk, p->ch, rt, 3);
-    if ((!three && p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch, rt, 2)) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
+    if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch, rt) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
     return HFRK_SUCCESS;
 }
 
-template <int MT, int WN, int WK, int CH, int RT, int NBUF, bool PACKED>
+template <int MT, int WN, int WK, int CH, int RT, bool PACKED>
 static int launch_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_kernel<MT, WN, WK, CH, RT, NBUF, PACKED>;
+    auto kern = skinny_gemm_kernel<MT, WN, WK, CH, RT, PACKED>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -707,13 +660,8 @@ static int launch_packing(const GemmArgs& args, int lds_bytes, hipStream_t strea
 
 template <int MT, int WN, int WK, int CH, int RT>
 static int launch_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    if constexpr (MT >= 2 && lds_bytes_for(MT, WK, CH, RT, 3) <= kLdsLimit) {
-        if (lds_bytes == lds_bytes_for(MT, WK, CH, RT, 3))
-            return args.packed ? launch_packing<MT, WN, WK, CH, RT, 3, true>(args, lds_bytes, stream)
-                               : launch_packing<MT, WN, WK, CH, RT, 3, false>(args, lds_bytes, stream);
-    }
-    return args.packed ? launch_packing<MT, WN, WK, CH, RT, 2, true>(args, lds_bytes, stream)
-                       : launch_packing<MT, WN, WK, CH, RT, 2, false>(args, lds_bytes, stream);
+    return args.packed ? launch_packing<MT, WN, WK, CH, RT, true>(args, lds_bytes, stream)
+                       : launch_packing<MT, WN, WK, CH, RT, false>(args, lds_bytes, stream);
 }
 
 template <int MT>

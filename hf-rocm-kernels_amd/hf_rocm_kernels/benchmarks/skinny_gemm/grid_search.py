@@ -44,12 +44,11 @@ def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.Gemm
             for g in grids:
                 plans.append(_capi.GemmPlan(mt, -1, wave_k // 256, 0, min(g, 256, tiles * windows), tiles, windows,
                                             8 * (wave_k // 256) * 4096 + 16 * mt * 1024))
-    # workgroup: row waves, chunks per slab, tiles per wave, staged activation slabs (three from 17 rows up)
-    for wn, ch, rt, nbuf in itertools.product((1, 2, 4, 8), (1, 2), (1, 2), (2, 3)):
+    for wn, ch, rt in itertools.product((1, 2, 4, 8), (1, 2), (1, 2)):  # workgroup: row waves, chunks per slab, tiles per wave
         wk = 8 // wn
         ks = 256 * wk * ch
-        lds = 8 * rt * 4096 + nbuf * 16 * mt * ks + (64 if nbuf == 3 else 16)
-        if k % ks or lds > 160 * 1024 or (rt == 2 and ch != 1) or (nbuf == 3 and mt < 2):
+        lds = 8 * rt * 4096 + 2 * 16 * mt * ks + 16
+        if k % ks or lds > 160 * 1024 or (rt == 2 and ch != 1):
             continue
         panels, slabs = -(-n // (16 * wn * rt)), k // ks
         for g in grids:
@@ -63,8 +62,7 @@ def describe(p: _capi.GemmPlan) -> str:
     if p.wn == -1:
         return f"k-split wave_k={256 * p.wk} windows={p.slabs} grid={p.grid}"
     tiles_per_wave = p.wn * p.wk // 8
-    slabs = 3 if (p.lds_bytes - 8 * tiles_per_wave * 4096) // (16 * p.m_tiles * 256 * p.wk * p.ch) == 3 else 2
-    return f"workgroup wn={p.wn // tiles_per_wave} wk={p.wk} ch={p.ch} rt={tiles_per_wave} bufs={slabs} grid={p.grid}"
+    return f"workgroup wn={p.wn // tiles_per_wave} wk={p.wk} ch={p.ch} rt={tiles_per_wave} grid={p.grid}"
 
 
 def time_plan(lib, arena: torch.Tensor, m: int, n: int, k: int, plan, reps: int, packed: bool = False) -> float:

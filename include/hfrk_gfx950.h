@@ -69,8 +69,7 @@ typedef struct hfrk_gemm_plan {
                       K-split: ceil(n/16) row tiles */
     int slabs;     /* workgroup: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per group.
                       K-split: k / (2048*wk) windows */
-    int lds_bytes; /* dynamic LDS per workgroup.  workgroup, m_tiles >= 2: 8*(wn*wk/8)*4096 + B*16*m_tiles*256*wk*ch + (B == 3 ? 64 : 16)
-                      with B = 2 staged activation slabs (a barrier per unit) or 3 (counters in LDS, waves run up to a unit apart) */
+    int lds_bytes; /* dynamic LDS per workgroup */
 } hfrk_gemm_plan;
 
 /* Library version, for the binding to check. */

@@ -76,15 +76,15 @@ def all_plans(m, n, k):
             ks = 256 * wk * ch
             if k % ks:
                 continue
+            lds = 8 * rt * 4096 + 2 * 16 * mt * ks + 16
+            if lds > 160 * 1024:
+                continue
             panels = (n + 16 * wn * rt - 1) // (16 * wn * rt)
             slabs = k // ks
             units = panels * slabs
-            for nbuf in ((2, 3) if mt >= 2 else (2,)):  # staged activation slabs: barrier hand-over, or three with counters
-                lds = 8 * rt * 4096 + nbuf * 16 * mt * ks + (64 if nbuf == 3 else 16)
-                if lds > 160 * 1024:
-                    continue
-                for grid in sorted({min(256, units), min(200, units), min(7, units)}):
-                    plans.append(_capi.GemmPlan(mt, wn * rt, wk, ch, grid, panels, slabs, lds))
+            for grid in sorted({min(256, units), min(200, units), min(7, units)}):
+                p = _capi.GemmPlan(mt, wn * rt, wk, ch, grid, panels, slabs, lds)
+                plans.append(p)
     return plans
 
 
