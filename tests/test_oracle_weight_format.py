@@ -86,3 +86,34 @@ def test_a_lane_operand_is_thirty_two_contiguous_k_bytes_of_one_row():
                 operand = np.concatenate([chunk[(2 * h) * 1024 + lane * 16:][:16], chunk[(2 * h + 1) * 1024 + lane * 16:][:16]])
                 c0 = kc * 256 + h * 128 + (lane // 16) * 32
                 assert np.array_equal(operand, w8[lane % 16, c0:c0 + 32])
+
+
+def test_pack_unpack_round_trip_on_random_shapes():
+    """Property check over many (n, k): unpack(pack(w)) == w, the packed size is the padded size, padding is zero."""
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=60, deadline=None)
+    @given(n=st.integers(1, 70), kc=st.integers(1, 3), seed=st.integers(0, 2 ** 31 - 1))
+    def check(n, kc, seed):
+        k = 256 * kc
+        w = np.random.default_rng(seed).integers(0, 256, (n, k), dtype=np.uint8)
+        packed = wf.pack_weight(w)
+        assert packed.size == wf.packed_bytes(n, k)
+        assert np.array_equal(wf.unpack_weight(packed, n, k), w)
+        assert int(packed.astype(np.int64).sum()) == int(w.astype(np.int64).sum())  # padding adds nothing
+        r, c = (seed % n), (seed // 7) % k
+        assert packed[wf.packed_offset(r, c, k)] == w[r, c]
+
+    check()
+
+
+def test_reencode_preserves_order_and_sign_symmetry():
+    """The code map is monotone in value (no two fnuz values swap order) and odd: map(-x) = -map(x)."""
+    fnuz, fn = wf.decode_table_fnuz(), fp8.decode_table()
+    table = wf.reencode_table()
+    codes = [c for c in range(256) if c != 0x80]
+    by_value = sorted(codes, key=lambda c: fnuz[c])
+    mapped = [fn[table[c]] for c in by_value]
+    assert all(a <= b for a, b in zip(mapped, mapped[1:]))
+    for c in range(1, 0x80):
+        assert fn[table[c | 0x80]] == -fn[table[c]]
