@@ -81,3 +81,41 @@ def llama_mlp_combined_ops(
     # Down projection
     skinny_gemm(skinny_a=swiglu_out, b=down_weight, scale_tensor=down_output_scale, output=mlp_output)
     return mlp_output, residual
+
+
+class LlamaMlpGraph:
+    """The decoder MLP sub-block captured once into a HIP graph: one host call per token step instead of three or four
+    operator launches (the reference times its kernels inside graphs, operators/skinny_gemm/benchmarking_fn.py:62-92,
+    but ships no captured block).
+
+    The graph reads `attn_output` and `residual` from buffers owned by this object: write the step's inputs with
+    `copy_` (or pass them to `__call__`, which does) and read the results from `mlp_output` / `residual`, which are
+    overwritten by every replay.  Weights and scales are the tensors given here; replace their contents in place if
+    they change.  Capturing needs the library's workspace to exist, so one eager run happens first."""
+
+    def __init__(self, rows: int, hidden: int, rms_weight: Tensor, rms_epsilon: float, gate_up_weight, gate_up_input_scale: Tensor,
+                 gate_up_output_scale: Tensor, down_weight, down_input_scale: Tensor, down_output_scale: Tensor,
+                 dtype: torch.dtype = torch.bfloat16, add_residual: bool = True, fused: bool = True):
+        device = rms_weight.device
+        self.attn_output = torch.zeros((rows, hidden), dtype=dtype, device=device)
+        self.residual = torch.zeros((rows, hidden), dtype=dtype, device=device)
+        args = (rms_weight, rms_epsilon, gate_up_weight, gate_up_input_scale, gate_up_output_scale, down_weight,
+                down_input_scale, down_output_scale)
+        kwargs = dict(add_residual=add_residual, fused=fused)
+        self._stream = torch.cuda.Stream(device)
+        with torch.cuda.stream(self._stream):
+            llama_mlp_combined_ops(self.attn_output, self.residual, *args, **kwargs)  # eager: workspace, code objects
+            self.residual.zero_()
+            torch.cuda.synchronize(device)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, stream=self._stream):
+                self.mlp_output, residual_out = llama_mlp_combined_ops(self.attn_output, self.residual, *args, **kwargs)
+        assert residual_out.data_ptr() == self.residual.data_ptr()  # updated in place
+        torch.cuda.synchronize(device)
+
+    def __call__(self, attn_output: Tensor, residual: Tensor) -> Tuple[Tensor, Tensor]:
+        """Copy the inputs in, replay, return (mlp_output, residual) -- views of this object's buffers."""
+        self.attn_output.copy_(attn_output)
+        self.residual.copy_(residual)
+        self.graph.replay()
+        return self.mlp_output, self.residual

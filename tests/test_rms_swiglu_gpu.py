@@ -252,3 +252,33 @@ def test_dynamic_ops_reject_rows_they_cannot_hold():
     assert rms(40000) == _capi.BAD_SHAPE       # wider than the register cache
     assert lib.hfrk_swiglu_dynamic(x.data_ptr(), q.data_ptr(), s.data_ptr(), None, 1, 20004, 0, _capi.BF16, None) == _capi.BAD_SHAPE
     assert lib.hfrk_swiglu_dynamic(x.data_ptr() + 2, q.data_ptr(), s.data_ptr(), None, 1, 64, 0, _capi.BF16, None) == _capi.BAD_ALIGNMENT
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_captured_mlp_block_replays_like_the_eager_block(packed):
+    """LlamaMlpGraph: the fused block as one graph launch.  Replayed several times with fresh inputs, with the
+    program's own eager launches and synchronisations in between; every replay must equal the eager result bit for bit."""
+    from hf_rocm_kernels.combined_ops.llama_mlp import LlamaMlpGraph, llama_mlp_combined_ops
+    from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    from hf_rocm_kernels.utils.weight_format import pack_weight
+    g = torch.Generator().manual_seed(5)
+    m, hidden, inter = 8, 1024, 2816
+    wn = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16).cuda()
+    wgu = (0.02 * torch.randn(2 * inter, hidden, generator=g)).cuda()
+    wd = (0.02 * torch.randn(hidden, inter, generator=g)).cuda()
+    qgu, sgu = fp8_quantize(wgu, amax_scale(wgu))
+    qd, sd = fp8_quantize(wd, amax_scale(wd))
+    w_gu = pack_weight(qgu) if packed else qgu.t()
+    w_d = pack_weight(qd) if packed else qd.t()
+    s_in, s_mid = torch.full((1,), 0.02, device="cuda"), torch.full((1,), 0.01, device="cuda")
+    args = (wn, 1e-5, w_gu, s_in, (s_in * sgu).view(1), w_d, s_mid, (s_mid * sd).view(1))
+    block = LlamaMlpGraph(m, hidden, *args)
+    for step in range(4):
+        x = torch.randn(m, hidden, generator=g).to(torch.bfloat16).cuda()
+        res = torch.randn(m, hidden, generator=g).to(torch.bfloat16).cuda()
+        want, want_res = llama_mlp_combined_ops(x, res.clone(), *args, add_residual=True, fused=True)
+        torch.cuda.synchronize()
+        got, got_res = block(x, res)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(got_res, want_res), step
+        assert got.float().abs().sum() > 0
