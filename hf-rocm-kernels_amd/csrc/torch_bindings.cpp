@@ -346,6 +346,17 @@ bool is_byte_tensor(const at::Tensor& t) {
     return t.scalar_type() == at::kByte || t.scalar_type() == at::kFloat8_e4m3fn || t.scalar_type() == at::kFloat8_e4m3fnuz;
 }
 
+// The fused GEMM for tracers: same call as skinny_gemm_fused / skinny_gemm_packed, but a status other than 0 raises
+// instead of being returned.  An operator that returns an integer cannot be part of a traced graph; one that returns
+// nothing can.
+void skinny_gemm_checked(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, at::Tensor& D, const std::optional<at::Tensor>& base,
+                         at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
+                         int64_t epilogue, int64_t intermediate_dtype) {
+    TORCH_CHECK(packed || B.dim() == 2, "B must be [k, n] with unit stride along k");
+    raise_on((int)gemm_fused_common(A, B, packed, packed ? n : B.size(1), D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype),
+             "skinny_gemm_checked");
+}
+
 // Row-major [n, k] fp8 weight -> packed load format; src_format 1 re-encodes e4m3fnuz values as e4m3fn on the way.
 void pack_weight(at::Tensor& src, at::Tensor& dst, int64_t src_format) {
     TORCH_CHECK(src.dim() == 2 && src.stride(1) == 1 && is_byte_tensor(src), "src must be a [n, k] one-byte tensor with unit stride along k");
@@ -411,6 +422,11 @@ TORCH_LIBRARY(_HFRK_C, ops) {
         "skinny_gemm_packed(Tensor A, Tensor B_packed, int n, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
         "Tensor? out_scale, int epilogue, int intermediate_dtype) -> int");
     ops.impl("skinny_gemm_packed", c10::kCUDA, &skinny_gemm_packed);
+
+    ops.def(
+        "skinny_gemm_checked(Tensor A, Tensor B, bool packed, int n, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
+        "Tensor? out_scale, int epilogue, int intermediate_dtype) -> ()");
+    ops.impl("skinny_gemm_checked", c10::kCUDA, &skinny_gemm_checked);
 
     ops.def("pack_weight(Tensor src, Tensor! dst, int src_format) -> ()");
     ops.impl("pack_weight", c10::kCUDA, &pack_weight);

@@ -10,6 +10,7 @@ from .operators.swiglu import swiglu, swiglu_dynamic
 from .operators.skinny_gemm import skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu
 from .operators.quantize import quantize_fp8
 
+from . import _fake_kernels  # noqa: F401  (shape-only implementations, so the operators can be traced)
 from . import plan_table
 
 plan_table.load_from_environment()  # HFRK_PLAN_TABLE=<json>: tuned GEMM decompositions, if the deployment has a table

@@ -41,3 +41,9 @@ def _skinny_gemm_fused(A: Tensor, B: Tensor, D: Tensor, base, scale_a: Tensor, s
 def _skinny_gemm_packed(A: Tensor, B_packed: Tensor, n: int, D: Tensor, base, scale_a: Tensor, scale_b, out_scale, epilogue: int,
                         intermediate_dtype: int) -> int:
     return torch.ops._HFRK_C.skinny_gemm_packed(A, B_packed, n, D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)
+
+
+def _skinny_gemm_checked(A: Tensor, B: Tensor, packed: bool, n: int, D: Tensor, base, scale_a: Tensor, scale_b, out_scale,
+                         epilogue: int, intermediate_dtype: int) -> None:
+    """The fused GEMM as an operator that raises instead of returning its status (traceable: it returns nothing)."""
+    torch.ops._HFRK_C.skinny_gemm_checked(A, B, packed, n, D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)

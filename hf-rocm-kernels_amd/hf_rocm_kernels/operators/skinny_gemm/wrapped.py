@@ -5,7 +5,7 @@ from torch import Tensor
 
 from ... import _capi
 from ...utils.weight_format import PackedWeight
-from .binding import _skinny_gemm, _skinny_gemm_fused, _skinny_gemm_packed, _skinny_gemm_scaled
+from .binding import _skinny_gemm, _skinny_gemm_checked, _skinny_gemm_fused, _skinny_gemm_packed, _skinny_gemm_scaled
 
 _OUT_DTYPES = (torch.bfloat16, torch.float16)
 
@@ -48,6 +48,13 @@ def infer_skinny_gemm_m_params(m: int) -> Tuple[int, int]:
     return a_lanes, op_m
 
 
+@torch.compiler.assume_constant_result
+def _planned_k_slabs(m: int, n: int, k: int) -> int:
+    """K slabs per row panel in the library's plan for the shape: a host-only call into the C library, a constant
+    of the shape to a tracer (which cannot follow a ctypes call)."""
+    return int(_capi.plan(m, n, k).slabs)
+
+
 def infer_skinny_gemm_params(skinny_a: Tensor, b: Tensor) -> Dict[str, int]:
     """The nine integers of the op schema.
 
@@ -61,10 +68,9 @@ def infer_skinny_gemm_params(skinny_a: Tensor, b: Tensor) -> Dict[str, int]:
     ops = 4 if op_m == 8 else 8
     b_lanes = min(4, max(1, n // (256 * 16)))
     qsize = 3
-    plan = _capi.plan(m, n, k)
     return {"A_producers": 3, "B_producers": min(6, qsize * b_lanes), "consumers": 3,
             "a_lanes": a_lanes, "b_lanes": b_lanes,
-            "qsize": qsize, "op_m": op_m, "ops": ops, "split_k": plan.slabs}
+            "qsize": qsize, "op_m": op_m, "ops": ops, "split_k": _planned_k_slabs(m, n, k)}
 
 
 def _raise_on_status(status: int, what: str) -> None:
@@ -75,7 +81,11 @@ def _raise_on_status(status: int, what: str) -> None:
 def _fused(skinny_a: Tensor, b, output: Tensor, base: Optional[Tensor], scale_a: Tensor, scale_b: Optional[Tensor],
            out_scale: Optional[Tensor], epilogue: int, intermediate_dtype: int) -> None:
     """One launch of the fused GEMM on a row-major view or a PackedWeight; raises on a non-zero status."""
-    if isinstance(b, PackedWeight):
+    if torch.compiler.is_compiling():  # an operator that returns its status cannot stay inside a traced graph
+        packed = isinstance(b, PackedWeight)
+        _skinny_gemm_checked(skinny_a, b.data if packed else b, packed, b.n if packed else b.size(1), output, base, scale_a,
+                             scale_b, out_scale, epilogue, intermediate_dtype)
+    elif isinstance(b, PackedWeight):
         status = _skinny_gemm_packed(skinny_a, b.data, b.n, output, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype)
         _raise_on_status(status, "skinny_gemm_packed")
     else:
@@ -104,7 +114,7 @@ def skinny_gemm(
     if output is None:
         output = torch.zeros(size=(skinny_a.size(0), b.size(1)), dtype=torch.bfloat16, device=skinny_a.device)
     skinny_gemm_checks(skinny_a, b, scale_tensor, output)
-    if isinstance(b, PackedWeight):  # the 13-argument op takes the row-major view only
+    if isinstance(b, PackedWeight) or torch.compiler.is_compiling():  # the 13-argument op takes the row-major view only
         _fused(skinny_a, b, output, output, scale_tensor.view(-1), None, None, _capi.EPILOGUE_NONE, 0)
         return output
     kwargs = infer_skinny_gemm_params(skinny_a, b)
@@ -130,7 +140,7 @@ def skinny_gemm_scaled(
     skinny_gemm_checks(skinny_a, b, scale_a.reshape(-1)[:1], output)
     assert scale_a.numel() in (1, m) and scale_a.dtype == torch.float32, f"Expected 1 or {m} float32 in scale_a"
     assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
-    if isinstance(b, PackedWeight):
+    if isinstance(b, PackedWeight) or torch.compiler.is_compiling():
         _fused(skinny_a, b, output, output if accumulate else None, scale_a.contiguous().view(-1), scale_b.contiguous().view(-1),
                None, _capi.EPILOGUE_NONE, 0)
         return output

@@ -76,7 +76,9 @@ typedef struct hfrk_gemm_plan {
 int hfrk_version(void);
 
 /* Allocate (once per device) the split-K workspace of the current device.  Idempotent, thread-safe.
- * Must have run on a device before a GEMM on that device is captured into a graph.  No reference counterpart
+ * Must have run on a device before a GEMM on that device is captured into a graph.  All GEMM launches on one
+ * device share this workspace and its arrival counters: order them on one stream (or one chain of graph nodes);
+ * two GEMMs running at the same time on one device would mix their partial sums.  No reference counterpart
  * (the reference accumulates with fp16 atomics into a caller-zeroed output instead of using a workspace). */
 int hfrk_init(void);
 

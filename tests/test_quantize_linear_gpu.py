@@ -130,3 +130,31 @@ def test_fp8_linear_module_tracks_the_float_layer_and_accepts_quantised_activati
     want = apply_fp8_linear(q, layer.weight, layer.weight_scale, scales, layer.bias)
     assert torch.equal(got, want) and got.dtype == torch.bfloat16
     assert "in_features=2048" in repr(layer)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_traced_fp8_linear_equals_the_eager_layer(packed):
+    """The layer traces as one graph (quantisation kernel and GEMM have shape-only implementations, and the GEMM
+    goes through the operator that raises instead of returning a status); traced and eager outputs are identical."""
+    from hf_rocm_kernels.layers import Fp8Linear
+    torch.manual_seed(1)
+    lin = torch.nn.Linear(1024, 768, bias=True).to(torch.bfloat16).cuda()
+    layer = Fp8Linear.from_float(lin, per_channel=True, packed=packed)
+    traced = torch.compile(layer, backend="aot_eager", fullgraph=True)
+    for rows in (1, 8, 8, 70):  # 70 rows: two GEMM launches of at most 64 rows
+        x = torch.randn(rows, 1024, device="cuda").to(torch.bfloat16)
+        assert torch.equal(traced(x), layer(x)), rows
+
+
+def test_checked_gemm_operator_raises_where_the_status_operator_returns_a_code():
+    import hf_rocm_kernels  # noqa: F401
+    a = torch.zeros(4, 512, device="cuda").to(torch.float8_e4m3fn)
+    w = torch.zeros(64, 512, device="cuda").to(torch.float8_e4m3fn)
+    one = torch.ones(1, device="cuda")
+    d = torch.zeros(4, 64, device="cuda", dtype=torch.bfloat16)
+    torch.ops._HFRK_C.skinny_gemm_checked(a, w.t(), False, 64, d, None, one, None, None, 0, 0)
+    bad_a = torch.zeros(4, 384, device="cuda").to(torch.float8_e4m3fn)  # k not a multiple of 256
+    bad_w = torch.zeros(64, 384, device="cuda").to(torch.float8_e4m3fn)
+    assert torch.ops._HFRK_C.skinny_gemm_fused(bad_a, bad_w.t(), d, None, one, None, None, 0, 0) == 3
+    with pytest.raises(RuntimeError, match="status 3"):
+        torch.ops._HFRK_C.skinny_gemm_checked(bad_a, bad_w.t(), False, 64, d, None, one, None, None, 0, 0)

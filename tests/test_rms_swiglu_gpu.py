@@ -282,3 +282,34 @@ def test_captured_mlp_block_replays_like_the_eager_block(packed):
         torch.cuda.synchronize()
         assert torch.equal(got, want) and torch.equal(got_res, want_res), step
         assert got.float().abs().sum() > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [False, True])
+def test_traced_mlp_block_equals_the_eager_block(fused):
+    """The operators have shape-only implementations, so torch can trace the block as one graph (no graph break) and
+    functionalise its in-place writes; the traced function must return what the eager one does, bit for bit."""
+    from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
+    from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    g = torch.Generator().manual_seed(6)
+    m, hidden, inter = 8, 1024, 2816
+    wn = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16).cuda()
+    wgu = (0.02 * torch.randn(2 * inter, hidden, generator=g)).cuda()
+    wd = (0.02 * torch.randn(hidden, inter, generator=g)).cuda()
+    qgu, sgu = fp8_quantize(wgu, amax_scale(wgu))
+    qd, sd = fp8_quantize(wd, amax_scale(wd))
+    s_in, s_mid = torch.full((1,), 0.02, device="cuda"), torch.full((1,), 0.01, device="cuda")
+    args = (wn, 1e-5, qgu.t(), s_in, (s_in * sgu).view(1), qd.t(), s_mid, (s_mid * sd).view(1))
+
+    def block(x, res):
+        return llama_mlp_combined_ops(x, res, *args, add_residual=True, fused=fused)
+
+    traced = torch.compile(block, backend="aot_eager", fullgraph=True)
+    for step in range(3):
+        x = torch.randn(m, hidden, generator=g).to(torch.bfloat16).cuda()
+        res = torch.randn(m, hidden, generator=g).to(torch.bfloat16).cuda()
+        want, want_res = block(x, res.clone())
+        got, got_res = traced(x, res.clone())
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(got_res, want_res), step
+        assert got.float().abs().sum() > 0
