@@ -14,7 +14,6 @@ Other workloads, same method, for the remaining configurations:
               (`skinny_gemm_scaled`, activation rows 1 and M-1 drawn 20x larger)
   mlp         the decoder MLP sub-block (`llama_mlp_combined_ops`: residual RMSNorm -> gate_up GEMM -> SwiGLU ->
               down GEMM, output added to the residual), hidden 4096, M in {1, 8, 16}: 3 blocks = 12 launches per step
-  mlp-block   the same block in ONE launch (`llama_mlp_block`: persistent kernel, phases behind grid-wide gates)
   mlp-fused   the same block in three launches: RMSNorm, gate_up GEMM with SwiGLU epilogue, down GEMM reading the
               residual as its addend (`llama_mlp_combined_ops(..., fused=True)`)
   pack        the step before the path: the four Llama-3-8B weights packed into the load format from float8_e4m3fn,
@@ -296,16 +295,13 @@ def make_mlp_inputs(torch, packed=False):
     return copies, acts, rms_w, s_in, s_mid
 
 
-def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused, one_launch=False):
-    from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_block, llama_mlp_combined_ops
+def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused):
+    from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
     out_scales = [((s_in * sgu).contiguous(), (s_mid * sd).contiguous()) for _, sgu, _, sd in copies]
 
     def call(m, ci):
         wgu, _, wd, _ = copies[ci]
         x, res = acts[m]
-        if one_launch:
-            return llama_mlp_block(x, res, rms_w, MLP["eps"], wgu, s_in, out_scales[ci][0], wd, s_mid, out_scales[ci][1],
-                                   add_residual=True)
         return llama_mlp_combined_ops(x, res, rms_w, MLP["eps"], wgu, s_in, out_scales[ci][0], wd, s_mid,
                                       out_scales[ci][1], add_residual=True, fused=fused)
     return call
@@ -467,7 +463,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "mlp-block", "pack"], default="llama3-8b")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "pack"], default="llama3-8b")
     ap.add_argument("--detail", action="store_true", help="also time every case on its own (HBM-cold and cache-hot)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--packed", action="store_true",
@@ -486,21 +482,17 @@ def main():
     if args.workload == "pack":
         print(json.dumps(run_pack_workload(torch, args)))
         return
-    is_mlp = args.workload in ("mlp", "mlp-fused", "mlp-block")
+    is_mlp = args.workload in ("mlp", "mlp-fused")
     if is_mlp:
         fused = args.workload == "mlp-fused"
-        one_launch = args.workload == "mlp-block"
         copies, acts, rms_w, s_in, s_mid = make_mlp_inputs(torch, args.packed)
-        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused, one_launch)
+        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused)
         graphs, keep = capture_mlp_steps(torch, call)
         step_bytes = sum(mlp_block_bytes(m) for m in MLP["ms"])
-        calls, text, metric = (1 if one_launch else 3 if fused else 4) * len(MLP["ms"]), MLP["text"], MLP["metric"]
+        calls, text, metric = (3 if fused else 4) * len(MLP["ms"]), MLP["text"], MLP["metric"]
         if fused:
             text = text.replace("3 blocks = 12 launches", "fused into 3 launches per block: 3 blocks = 9 launches")
-        if one_launch:
-            text = text.replace("3 blocks = 12 launches", "one persistent kernel per block: 3 blocks = 3 launches")
-        kernel = ("llama_mlp_block_kernel" if one_launch else
-                  "residual_rms_vec_kernel + skinny_gemm_stream_kernel<MA,2,swiglu> + skinny_gemm_stream_kernel" if fused else
+        kernel = ("residual_rms_vec_kernel + skinny_gemm_stream_kernel<MA,2,swiglu> + skinny_gemm_stream_kernel" if fused else
                   "residual_rms_vec_kernel + skinny_gemm_stream_kernel + swiglu_vec_kernel + skinny_gemm_stream_kernel")
         n_copies = MLP["cycle"]
     else:

@@ -12,11 +12,28 @@
 //   16-bit output:  round16( float(round16(float(z) * r)) * float(weight) )
 //   fp8 output:     e4m3fn( clamp( float(z) * r * float(weight) * (1/scale), +-448 ) )   no 16-bit detour, as in
 //                   the reference's vectorised kernel (residual_rms_vectorized.cu:124-135)
-#include "residual_rms_row.h"
+#include "hfrk_internal.h"
 
 namespace hfrk {
 
 constexpr int kRmsMaxThreads = 1024;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// Sum over the workgroup; every thread returns the same bits.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6, nwaves = (blockDim.x + 63) >> 6;
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < nwaves; ++w) total += red[w];
+    return total;
+}
 
 __device__ __forceinline__ void zero_next_buffer_row(uint16_t* next_buffer, int buffer_cols) {
     if (buffer_cols <= 0) return;
@@ -39,7 +56,76 @@ __global__ void __launch_bounds__(kRmsMaxThreads) residual_rms_vec_kernel(
     const float* __restrict__ scale_tensor, void* __restrict__ output, uint16_t* __restrict__ next_buffer,
     float epsilon, int cols, int buffer_cols) {
     __shared__ float red[16];
-    rms_row_vec<DT, FP8_OUT, ITERS, false>(input, residual, weight, scale_tensor, output, epsilon, cols, (int)blockIdx.x, red);
+    const long row_off = (long)blockIdx.x * cols;
+    const int nvec = cols >> 3;
+    uint4 z[ITERS], wreg[ITERS];
+    float ssq = 0.f;
+    // Everything the second pass needs is requested now, so that the kernel pays one memory latency, not two.
+    float scale = 1.f;
+    if constexpr (FP8_OUT) scale = scale_tensor[0];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = threadIdx.x + it * blockDim.x;
+        wreg[it] = make_uint4(0, 0, 0, 0);
+        if (v < nvec) wreg[it] = reinterpret_cast<const uint4*>(weight)[v];
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = threadIdx.x + it * blockDim.x;
+        if (v < nvec) {
+            const uint4 a = reinterpret_cast<const uint4*>(input + row_off)[v];
+            const uint4 r = reinterpret_cast<const uint4*>(residual + row_off)[v];
+            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, rw[4] = {r.x, r.y, r.z, r.w};
+            uint32_t zw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint16_t lo = store16<DT>(load16<DT>((uint16_t)(aw[j] & 0xffff)) + load16<DT>((uint16_t)(rw[j] & 0xffff)));
+                const uint16_t hi = store16<DT>(load16<DT>((uint16_t)(aw[j] >> 16)) + load16<DT>((uint16_t)(rw[j] >> 16)));
+                const float fl = load16<DT>(lo), fh = load16<DT>(hi);
+                ssq += fl * fl;
+                ssq += fh * fh;
+                zw[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            z[it] = make_uint4(zw[0], zw[1], zw[2], zw[3]);
+            reinterpret_cast<uint4*>(residual + row_off)[v] = z[it];
+        }
+    }
+    const float total = block_sum(ssq, red);
+    const float norm = rsqrtf(total / (float)cols + epsilon);
+    const float inv_scale = 1.f / scale;
+
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int v = threadIdx.x + it * blockDim.x;
+        if (v < nvec) {
+            const uint4 w = wreg[it];
+            const uint32_t zw[4] = {z[it].x, z[it].y, z[it].z, z[it].w}, ww[4] = {w.x, w.y, w.z, w.w};
+            if constexpr (FP8_OUT) {
+                float y[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    y[2 * j] = load16<DT>((uint16_t)(zw[j] & 0xffff)) * norm * load16<DT>((uint16_t)(ww[j] & 0xffff)) * inv_scale;
+                    y[2 * j + 1] = load16<DT>((uint16_t)(zw[j] >> 16)) * norm * load16<DT>((uint16_t)(ww[j] >> 16)) * inv_scale;
+                }
+                uint32_t p0 = cvt_pk_fp8(y[0], y[1], 0u, false);
+                p0 = cvt_pk_fp8(y[2], y[3], p0, true);
+                uint32_t p1 = cvt_pk_fp8(y[4], y[5], 0u, false);
+                p1 = cvt_pk_fp8(y[6], y[7], p1, true);
+                reinterpret_cast<uint2*>(static_cast<uint8_t*>(output) + row_off)[v] = make_uint2(p0, p1);
+            } else {
+                uint32_t ow[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint16_t nl = store16<DT>(load16<DT>((uint16_t)(zw[j] & 0xffff)) * norm);
+                    const uint16_t nh = store16<DT>(load16<DT>((uint16_t)(zw[j] >> 16)) * norm);
+                    const uint16_t ol = store16<DT>(load16<DT>(nl) * load16<DT>((uint16_t)(ww[j] & 0xffff)));
+                    const uint16_t oh = store16<DT>(load16<DT>(nh) * load16<DT>((uint16_t)(ww[j] >> 16)));
+                    ow[j] = (uint32_t)ol | ((uint32_t)oh << 16);
+                }
+                reinterpret_cast<uint4*>(static_cast<uint16_t*>(output) + row_off)[v] = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+            }
+        }
+    }
     zero_next_buffer_row(next_buffer, buffer_cols);
 }
 

@@ -441,10 +441,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 // ------------------------------------------------------------------------------------------------------------
 struct DeviceState {
     float* ws = nullptr;
-    int* counters = nullptr;   // kMaxPanels arrival counters, then kGateWords words for the MLP block's gates
-    int num_cu = 0;
+    int* counters = nullptr;
 };
-constexpr int kGateWords = 64;
 static DeviceState g_dev[64];
 static std::mutex g_mutex;
 
@@ -467,10 +465,8 @@ static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
         float* ws = nullptr;
         int* counters = nullptr;
         HFRK_HIP_TRY(hipMalloc(&ws, kWsFloats * sizeof(float)));
-        hipError_t e = hipMalloc(&counters, (kMaxPanels + kGateWords) * sizeof(int));
-        if (e == hipSuccess) e = hipMemset(counters, 0, (kMaxPanels + kGateWords) * sizeof(int));
-        int num_cu = 0;
-        if (e == hipSuccess) e = hipDeviceGetAttribute(&num_cu, hipDeviceAttributeMultiprocessorCount, dev);
+        hipError_t e = hipMalloc(&counters, kMaxPanels * sizeof(int));
+        if (e == hipSuccess) e = hipMemset(counters, 0, kMaxPanels * sizeof(int));
         if (e != hipSuccess) {
             (void)hipFree(ws);
             if (counters) (void)hipFree(counters);
@@ -478,7 +474,6 @@ static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
             return HFRK_HIP_ERROR;
         }
         g_dev[dev].counters = counters;
-        g_dev[dev].num_cu = num_cu;
         g_dev[dev].ws = ws;
     }
     *out = &g_dev[dev];
@@ -789,108 +784,9 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     return HFRK_INVALID_CONFIG;
 }
 
-// One GemmArgs of the MLP block: a wave-stream plan on a grid of kNumCU, row_tiles 2 with the SwiGLU epilogue.
-static int fill_block_gemm(GemmArgs* g, const void* A, const void* B, void* D, const void* base, const float* out_scale,
-                           const float* scale, int m, int n, int k, bool swiglu, bool packed, int d_dtype, DeviceState* st) {
-    if (((long)n + 128) * k + k >= (1L << 31)) return HFRK_BAD_SHAPE;
-    hfrk_gemm_plan p;
-    const int rc = fill_stream_plan(m, swiglu ? n / 2 : n, k, 1, false, kNumCU, &p);
-    if (rc != HFRK_SUCCESS) return rc;
-    if (p.grid != kNumCU) return HFRK_BAD_SHAPE;  // fewer chunks than workgroups
-    g->A = static_cast<const uint8_t*>(A);
-    g->B = static_cast<const uint8_t*>(B);
-    g->D = D;
-    g->base = base;
-    g->out_scale = out_scale;
-    g->scale_a = scale;
-    g->scale_b = nullptr;
-    g->sa_stride = 0;
-    g->sb_stride = 0;
-    g->m = m;
-    g->n = n;
-    g->k = k;
-    g->b_stride = k;
-    g->packed = packed ? 1 : 0;
-    g->d_dtype = d_dtype;
-    g->panels = p.panels;
-    g->slabs = p.slabs;
-    g->units = p.panels * p.slabs;
-    g->grid = p.grid;
-    g->chunks_q = g->units / p.grid;
-    g->chunks_r = g->units % p.grid;
-    g->ws = st->ws;
-    g->counters = st->counters;
-    return HFRK_SUCCESS;
-}
-
-static int mlp_block_launch(const void* input, void* residual, const void* rms_weight, float epsilon, const void* gate_up_weight,
-                            const float* gate_up_input_scale, const float* gate_up_output_scale, const void* down_weight,
-                            const float* down_input_scale, const float* down_output_scale, void* normalized, void* activated,
-                            void* output, int m, int hidden, int inter, int io_dtype, int packed, int add_residual,
-                            int spin_limit, hipStream_t stream) {
-    if (m < 1 || m > 16 || hidden < 256 || inter < 256) return HFRK_BAD_SHAPE;
-    if (hidden % 256 != 0 || inter % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
-    if (hidden > 8 * kGemmThreads * 2) return HFRK_BAD_SHAPE;  // a row is normalised by 512 threads, two vectors each at most
-    if (io_dtype != HFRK_F16 && io_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
-    if (!input || !residual || !rms_weight || !gate_up_weight || !gate_up_input_scale || !gate_up_output_scale || !down_weight ||
-        !down_input_scale || !down_output_scale || !normalized || !activated || !output)
-        return HFRK_BAD_SHAPE;
-    if (!(epsilon > 0.f) || spin_limit < 1) return HFRK_INVALID_CONFIG;
-    const uintptr_t all = reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(rms_weight) |
-                          reinterpret_cast<uintptr_t>(gate_up_weight) | reinterpret_cast<uintptr_t>(down_weight) |
-                          reinterpret_cast<uintptr_t>(normalized) | reinterpret_cast<uintptr_t>(activated) | reinterpret_cast<uintptr_t>(output);
-    if (all & 15) return HFRK_BAD_ALIGNMENT;
-
-    int dev = 0;
-    HFRK_HIP_TRY(hipGetDevice(&dev));
-    DeviceState* st = nullptr;
-    int rc = ensure_workspace(dev, stream, &st);
-    if (rc != HFRK_SUCCESS) return rc;
-    if (st->num_cu < kNumCU) return HFRK_INVALID_CONFIG;  // the gates need every workgroup resident, one per CU
-
-    MlpBlockArgs args;
-    args.input = static_cast<const uint16_t*>(input);
-    args.residual = static_cast<uint16_t*>(residual);
-    args.rms_weight = static_cast<const uint16_t*>(rms_weight);
-    args.rms_scale = gate_up_input_scale;
-    args.normalized = static_cast<uint8_t*>(normalized);
-    args.epsilon = epsilon;
-    args.hidden = hidden;
-    args.io_dtype = io_dtype;
-    args.spin_limit = spin_limit;
-    args.bar = reinterpret_cast<unsigned*>(st->counters + kMaxPanels);
-    rc = fill_block_gemm(&args.gate_up, normalized, gate_up_weight, activated, nullptr, down_input_scale, gate_up_output_scale,
-                         m, 2 * inter, hidden, true, packed != 0, io_dtype, st);
-    if (rc != HFRK_SUCCESS) return rc;
-    rc = fill_block_gemm(&args.down, activated, down_weight, output, add_residual ? residual : nullptr, nullptr, down_output_scale,
-                         m, hidden, inter, false, packed != 0, io_dtype, st);
-    if (rc != HFRK_SUCCESS) return rc;
-    return launch_mlp_block_kernel(args, (m + 3) / 4, stream);
-}
-
 }  // namespace hfrk
 
 extern "C" {
-
-int hfrk_llama_mlp_block(const void* input, void* residual, const void* rms_weight, float epsilon, const void* gate_up_weight,
-                         const float* gate_up_input_scale, const float* gate_up_output_scale, const void* down_weight,
-                         const float* down_input_scale, const float* down_output_scale, void* normalized, void* activated,
-                         void* output, int m, int hidden, int inter, int io_dtype, int packed, int add_residual, void* stream) {
-    return hfrk::mlp_block_launch(input, residual, rms_weight, epsilon, gate_up_weight, gate_up_input_scale, gate_up_output_scale,
-                                  down_weight, down_input_scale, down_output_scale, normalized, activated, output, m, hidden, inter,
-                                  io_dtype, packed, add_residual, 1 << 16, static_cast<hipStream_t>(stream));
-}
-
-int hfrk_llama_mlp_block_timeouts(unsigned* count) {
-    if (!count) return HFRK_BAD_SHAPE;
-    int dev = 0;
-    HFRK_HIP_TRY(hipGetDevice(&dev));
-    hfrk::DeviceState* st = nullptr;
-    const int rc = hfrk::ensure_workspace(dev, nullptr, &st);
-    if (rc != HFRK_SUCCESS) return rc;
-    HFRK_HIP_TRY(hipMemcpy(count, st->counters + hfrk::kMaxPanels + 1, sizeof(unsigned), hipMemcpyDeviceToHost));
-    return HFRK_SUCCESS;
-}
 
 int hfrk_init(void) {
     int dev = 0;

@@ -46,24 +46,6 @@ constexpr bool stream_variant_exists(int act_loads, int row_tiles, bool swiglu =
                   : (row_tiles == 1 && act_loads >= 1 && act_loads <= 4) || (row_tiles == 2 && act_loads >= 3 && act_loads <= 8);
 }
 
-// Single-launch MLP block (llama_mlp_block.hip): residual RMSNorm, then the wave-stream GEMM twice (gate_up with the
-// SwiGLU epilogue, down with the residual as addend) behind grid-wide gates.  Both GEMMs run on a grid of kNumCU.
-struct MlpBlockArgs {
-    const uint16_t* input;       // [m, hidden] 16-bit
-    uint16_t* residual;          // [m, hidden] 16-bit, updated in place
-    const uint16_t* rms_weight;  // [hidden]
-    const float* rms_scale;      // quantisation scale of the normalised activations
-    uint8_t* normalized;         // [m, hidden] fp8: RMSNorm output, gate_up's activations
-    float epsilon;
-    int hidden;
-    int io_dtype;
-    int spin_limit;              // polls a workgroup spends at a gate before it gives up
-    unsigned* bar;               // [0] arrival counter, [1] time-outs
-    GemmArgs gate_up;            // A = normalized, D = the fp8 [m, inter] activations of the down GEMM
-    GemmArgs down;               // A = gate_up.D, base = residual or null, D = the block's output
-};
-int launch_mlp_block_kernel(const MlpBlockArgs& args, int act_loads, hipStream_t stream);
-
 // K-split kernel (skinny_gemm_ksplit.hip): the 8 waves of a workgroup split a K window of 8*wave_k bytes
 // (wave_k = 256, 512, or 1024 with m_tiles <= 2), activations in registers.  Needs k % (8*wave_k) == 0.
 int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, int lds_bytes, hipStream_t stream);

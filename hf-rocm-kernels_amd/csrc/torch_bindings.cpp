@@ -342,59 +342,6 @@ int64_t skinny_gemm_packed(at::Tensor& A, at::Tensor& B_packed, int64_t n, at::T
     return gemm_fused_common(A, B_packed, true, n, D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype);
 }
 
-// The decoder MLP sub-block in one launch (hfrk_llama_mlp_block): RMSNorm, gate_up GEMM + SwiGLU, down GEMM
-// (+ residual).  Counterpart of the launch sequence of the reference's combined_ops/llama_mlp.py:7-60 as one op.
-// Weights: the [k, n] views of contiguous row-major [n, k] tensors, or (packed) the buffers pack_weight wrote.
-// normalized [m, hidden] and activated [m, inter] are fp8 scratch the caller provides; output [m, hidden].
-void llama_mlp_block(at::Tensor& input, at::Tensor& residual, at::Tensor& rms_weight, double epsilon, at::Tensor& gate_up_weight,
-                     at::Tensor& gate_up_input_scale, at::Tensor& gate_up_output_scale, at::Tensor& down_weight,
-                     at::Tensor& down_input_scale, at::Tensor& down_output_scale, at::Tensor& normalized, at::Tensor& activated,
-                     at::Tensor& output, bool packed, int64_t inter, bool add_residual) {
-    TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous [m, hidden] tensor");
-    const int64_t m = input.size(0), hidden = input.size(1);
-    const int io = dtype16(input, "input");
-    TORCH_CHECK(m >= 1 && m <= 16 && hidden < (int64_t(1) << 20) && inter >= 1 && inter < (int64_t(1) << 20), "m must be 1..16; hidden and inter below 2^20");
-    for (const at::Tensor* t : {&residual, &output})
-        TORCH_CHECK(t->sizes() == input.sizes() && t->is_contiguous() && t->scalar_type() == input.scalar_type(),
-                    "residual and output must be contiguous tensors with input's shape and dtype");
-    TORCH_CHECK(rms_weight.dim() == 1 && rms_weight.size(0) == hidden && rms_weight.is_contiguous() && rms_weight.scalar_type() == input.scalar_type(),
-                "rms_weight must be a contiguous [hidden] tensor with input's dtype");
-    check_fp8(gate_up_weight, "gate_up_weight");
-    check_fp8(down_weight, "down_weight");
-    check_fp8(normalized, "normalized");
-    check_fp8(activated, "activated");
-    if (packed) {
-        TORCH_CHECK(gate_up_weight.is_contiguous() && (size_t)gate_up_weight.numel() == hfrk_packed_weight_bytes((int)(2 * inter), (int)hidden),
-                    "gate_up_weight must be the packed buffer of a [2*inter, hidden] weight");
-        TORCH_CHECK(down_weight.is_contiguous() && (size_t)down_weight.numel() == hfrk_packed_weight_bytes((int)hidden, (int)inter),
-                    "down_weight must be the packed buffer of a [hidden, inter] weight");
-    } else {
-        TORCH_CHECK(gate_up_weight.dim() == 2 && gate_up_weight.size(0) == hidden && gate_up_weight.size(1) == 2 * inter &&
-                        gate_up_weight.stride(0) == 1 && gate_up_weight.stride(1) == hidden,
-                    "gate_up_weight must be the [hidden, 2*inter] view of a contiguous [2*inter, hidden] tensor");
-        TORCH_CHECK(down_weight.dim() == 2 && down_weight.size(0) == inter && down_weight.size(1) == hidden &&
-                        down_weight.stride(0) == 1 && down_weight.stride(1) == inter,
-                    "down_weight must be the [inter, hidden] view of a contiguous [hidden, inter] tensor");
-    }
-    TORCH_CHECK(normalized.is_contiguous() && normalized.dim() == 2 && normalized.size(0) == m && normalized.size(1) == hidden,
-                "normalized must be a contiguous fp8 [m, hidden] tensor");
-    TORCH_CHECK(activated.is_contiguous() && activated.dim() == 2 && activated.size(0) == m && activated.size(1) == inter,
-                "activated must be a contiguous fp8 [m, inter] tensor");
-    for (const at::Tensor* t : {&gate_up_input_scale, &gate_up_output_scale, &down_input_scale, &down_output_scale}) {
-        TORCH_CHECK(t->scalar_type() == at::kFloat && t->numel() == 1, "the four scales must be one float32 each");
-        check_same_device(input, *t, "scale");
-    }
-    for (const at::Tensor* t : {&residual, &rms_weight, &gate_up_weight, &down_weight, &normalized, &activated, &output})
-        check_same_device(input, *t, "operand");
-    DeviceScope scope(input);
-    raise_on(hfrk_llama_mlp_block(input.data_ptr(), residual.data_ptr(), rms_weight.data_ptr(), (float)epsilon, gate_up_weight.data_ptr(),
-                                  gate_up_input_scale.data_ptr<float>(), gate_up_output_scale.data_ptr<float>(), down_weight.data_ptr(),
-                                  down_input_scale.data_ptr<float>(), down_output_scale.data_ptr<float>(), normalized.data_ptr(),
-                                  activated.data_ptr(), output.data_ptr(), (int)m, (int)hidden, (int)inter, io, packed ? 1 : 0,
-                                  add_residual ? 1 : 0, current_stream(input)),
-             "llama_mlp_block");
-}
-
 bool is_byte_tensor(const at::Tensor& t) {
     return t.scalar_type() == at::kByte || t.scalar_type() == at::kFloat8_e4m3fn || t.scalar_type() == at::kFloat8_e4m3fnuz;
 }
@@ -480,13 +427,6 @@ TORCH_LIBRARY(_HFRK_C, ops) {
         "skinny_gemm_checked(Tensor A, Tensor B, bool packed, int n, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
         "Tensor? out_scale, int epilogue, int intermediate_dtype) -> ()");
     ops.impl("skinny_gemm_checked", c10::kCUDA, &skinny_gemm_checked);
-
-    ops.def(
-        "llama_mlp_block(Tensor input, Tensor! residual, Tensor rms_weight, float epsilon, Tensor gate_up_weight, "
-        "Tensor gate_up_input_scale, Tensor gate_up_output_scale, Tensor down_weight, Tensor down_input_scale, "
-        "Tensor down_output_scale, Tensor! normalized, Tensor! activated, Tensor! output, bool packed, int inter, "
-        "bool add_residual) -> ()");
-    ops.impl("llama_mlp_block", c10::kCUDA, &llama_mlp_block);
 
     ops.def("pack_weight(Tensor src, Tensor! dst, int src_format) -> ()");
     ops.impl("pack_weight", c10::kCUDA, &pack_weight);

@@ -74,8 +74,6 @@ SIGNATURES = {
     "hfrk_residual_rms_dynamic": (_i, [_p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _p]),
     "hfrk_swiglu_dynamic": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
     "hfrk_quantize_fp8": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
-    "hfrk_llama_mlp_block": (_i, [_p, _p, _p, _f] + [_p] * 9 + [_i] * 6 + [_p]),
-    "hfrk_llama_mlp_block_timeouts": (_i, [ctypes.POINTER(ctypes.c_uint)]),
 }
 
 _lib = None

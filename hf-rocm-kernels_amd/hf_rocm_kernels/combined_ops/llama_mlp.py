@@ -83,45 +83,6 @@ def llama_mlp_combined_ops(
     return mlp_output, residual
 
 
-def llama_mlp_block(
-    attn_output: Tensor,
-    residual: Tensor,
-    rms_weight: Tensor,
-    rms_epsilon: float,
-    gate_up_weight,
-    gate_up_input_scale: Tensor,
-    gate_up_output_scale: Tensor,
-    down_weight,
-    down_input_scale: Tensor,
-    down_output_scale: Tensor,
-    add_residual: bool = True,
-    output: Optional[Tensor] = None,
-    scratch: Optional[Tuple[Tensor, Tensor]] = None,
-) -> Tuple[Tensor, Tensor]:
-    """The block of `llama_mlp_combined_ops(..., fused=True)` as ONE kernel launch (m <= 16): RMSNorm, gate_up GEMM with
-    the SwiGLU epilogue and down GEMM run as phases of one persistent kernel, separated by grid-wide gates across which
-    the weight stream keeps running.  Same arguments and results as the chain (reference: combined_ops/llama_mlp.py:7-60);
-    the weights are col-major views of contiguous [n, k] tensors, or both PackedWeight.
-    - output: optional (m, hidden) tensor for the result; scratch: optional (fp8 (m, hidden), fp8 (m, inter)) pair for the
-      two intermediate activations (allocated when omitted; they hold the intermediates afterwards)
-    Returns (mlp_output, residual)."""
-    from ..utils.weight_format import PackedWeight
-    m, hidden = attn_output.shape
-    packed = isinstance(gate_up_weight, PackedWeight)
-    assert packed == isinstance(down_weight, PackedWeight), "Expected both weights packed or both row-major views"
-    inter = (gate_up_weight.n if packed else gate_up_weight.size(1)) // 2
-    if output is None:
-        output = torch.empty_like(attn_output)
-    if scratch is None:
-        scratch = (torch.empty((m, hidden), dtype=torch.float8_e4m3fn, device=attn_output.device),
-                   torch.empty((m, inter), dtype=torch.float8_e4m3fn, device=attn_output.device))
-    torch.ops._HFRK_C.llama_mlp_block(
-        attn_output, residual, rms_weight, rms_epsilon, gate_up_weight.data if packed else gate_up_weight, gate_up_input_scale,
-        gate_up_output_scale, down_weight.data if packed else down_weight, down_input_scale, down_output_scale, scratch[0],
-        scratch[1], output, packed, inter, add_residual)
-    return output, residual
-
-
 class LlamaMlpGraph:
     """The decoder MLP sub-block captured once into a HIP graph: one host call per token step instead of three or four
     operator launches (the reference times its kernels inside graphs, operators/skinny_gemm/benchmarking_fn.py:62-92,

@@ -147,30 +147,6 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
                            const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k,
                            int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
 
-/* The decoder MLP sub-block in ONE launch: residual <- input + residual; normalized = fp8(rmsnorm(residual) * rms_weight
- * / gate_up_input_scale); activated = fp8(silu(gate) * up / down_input_scale) with (gate, up) = gate_up_output_scale x
- * normalized x gate_up_weight^T rounded to io_dtype; output = (add_residual ? residual : 0) + down_output_scale x
- * activated x down_weight^T, rounded once.  Replaces the four launches of the reference's
- * hf_rocm_kernels/combined_ops/llama_mlp.py:7-60 (residual_rms, skinny_gemm, swiglu, skinny_gemm); same bits as
- * hfrk_residual_rms, hfrk_skinny_gemm_fused (SwiGLU epilogue) and hfrk_skinny_gemm_fused (base = residual) run one
- * after the other with wave-stream plans on a grid of 256.
- *   input, residual, output: [m, hidden] io_dtype (HFRK_F16 / HFRK_BF16); rms_weight [hidden] io_dtype; m <= 16
- *   gate_up_weight [2*inter, hidden], down_weight [hidden, inter]: fp8 row-major contiguous, or both packed (packed != 0)
- *   the four scales: one float each (per-tensor), as in the reference's chain
- *   normalized [m, hidden], activated [m, inter]: fp8 scratch of the caller, holding the intermediate results afterwards
- *   hidden, inter: multiples of 256; hidden <= 8192; every pointer 16-byte aligned
- * 256 workgroups that wait for one another at two grid-wide gates: the device must have 256 CUs, and nothing else
- * should occupy them for long while the launch runs.  The wait is bounded; a launch that gave up at a gate leaves
- * wrong results and raises the count hfrk_llama_mlp_block_timeouts reports.  Shares the GEMM workspace (stream order). */
-int hfrk_llama_mlp_block(const void* input, void* residual, const void* rms_weight, float epsilon, const void* gate_up_weight,
-                         const float* gate_up_input_scale, const float* gate_up_output_scale, const void* down_weight,
-                         const float* down_input_scale, const float* down_output_scale, void* normalized, void* activated,
-                         void* output, int m, int hidden, int inter, int io_dtype, int packed, int add_residual, void* stream);
-
-/* Gates of hfrk_llama_mlp_block that were abandoned on the current device since hfrk_init (0 in a healthy process).
- * `count` is a HOST pointer; this call synchronises with the device. */
-int hfrk_llama_mlp_block_timeouts(unsigned* count);
-
 /* Weight load format (no reference counterpart: the reference streams row-major weights through an LDS ring,
  * csrc/op_src/skinny_gemm/producers/n_full_tiles.cu:4-127, and stores fn bits viewed as fnuz,
  * hf_rocm_kernels/utils/fp8.py:27-29).  A weight packed once when the model is loaded is read by the GEMM as one
