@@ -691,15 +691,22 @@ static bool plan_key(int m, int n, int k, int packed, uint64_t* key) {
     return true;
 }
 
-// the tuned plan if there is one, else the planner's
+// The tuned plan if there is one, else the planner's.  An entry tuned for m' also serves every m below it that runs the
+// same kernel instance on the same work: for m <= 16 the same number of 4-row activation loads (m' = 8 serves 5..8),
+// above that the same number of 16-row tiles (m' = 32 serves 17..32); rows past m are out of the buffer's range and
+// cost no traffic.  The nearest such entry wins.
 static int choose_plan(int m, int n, int k, bool packed, hfrk_gemm_plan* plan) {
     uint64_t key;
     if (plan_key(m, n, k, packed, &key)) {
+        const int top = m <= 16 ? (m + 3) / 4 * 4 : (m + 15) / 16 * 16;
         std::lock_guard<std::mutex> lock(g_plan_mutex);
-        const auto it = g_plan_table.find(key);
-        if (it != g_plan_table.end()) {
-            *plan = it->second;
-            return HFRK_SUCCESS;
+        for (int mm = m; mm <= top && !g_plan_table.empty(); ++mm) {
+            if (!plan_key(mm, n, k, packed, &key)) break;
+            const auto it = g_plan_table.find(key);
+            if (it != g_plan_table.end() && check_plan(m, n, k, false, &it->second) == HFRK_SUCCESS) {
+                *plan = it->second;
+                return HFRK_SUCCESS;
+            }
         }
     }
     return make_plan(m, n, k, plan);

@@ -98,8 +98,10 @@ int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, in
  * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102).  Returns HFRK_SUCCESS or a shape error. */
 int hfrk_skinny_gemm_plan(int m, int n, int k, hfrk_gemm_plan* plan);
 
-/* Plan table (host only, thread-safe): tuned decompositions that take the planner's place for exact keys
- * (m, n, k, packed) whenever a GEMM entry point is called without a plan (the SwiGLU epilogue keeps its own plan).
+/* Plan table (host only, thread-safe): tuned decompositions, keyed (m, n, k, packed), that take the planner's place
+ * whenever a GEMM entry point is called without a plan (the SwiGLU epilogue keeps its own plan).  An entry also serves
+ * the smaller m that run the same kernel on the same work: m' <= 16 serves m > m' - 4 rounded to fours (8 serves 5..8),
+ * m' > 16 serves down to the previous multiple of 16 (32 serves 17..32); the nearest entry at or above m wins.
  * Counterpart of the reference's tuned table, hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102, filled from
  * sweeps like its benchmarks/skinny_gemm/grid_search.py.
  *   hfrk_plan_table_set    validates the plan for the shape like hfrk_skinny_gemm_ex does and stores it; plan == NULL

@@ -423,9 +423,13 @@ def test_a_plan_table_entry_is_what_a_call_without_a_plan_runs():
         assert plan_table.get_plan(m, n, k).as_dict() == entry.as_dict()
         after = skinny_gemm_scaled(a, b, sa, sw)
         after_packed = skinny_gemm_scaled(a, pack_weight(b.t()), sa, sw)
+        # the entry also serves m = 5..7 (same activation loads): same plan, first rows of the same product
+        assert plan_table.get_plan(6, n, k).as_dict() == entry.as_dict()
+        six = skinny_gemm_scaled(a[:6].contiguous(), b, sa, sw)
     finally:
         plan_table.clear()
         plan_table.load_from_environment()
     assert torch.equal(after, explicit) and torch.equal(after_packed, explicit)
+    assert torch.equal(six, explicit[:6])
     check_against_oracle(after, a, b, sa, sw)
     check_against_oracle(before, a, b, sa, sw)

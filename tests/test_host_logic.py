@@ -310,7 +310,7 @@ def test_bench_table_bookkeeping():
 
 
 def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_path, monkeypatch):
-    """hfrk_plan_table_* are host functions: entries replace the planner's choice for their exact key, invalid plans
+    """hfrk_plan_table_* are host functions: entries replace the planner's choice for their key (and the smaller m of the same bucket), invalid plans
     are refused with the launcher's status, and a table survives save -> clear -> load (also via HFRK_PLAN_TABLE)."""
     from hf_rocm_kernels import plan_table
     plan_table.clear()
@@ -323,7 +323,24 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
     assert plan_table.get_plan(m, n, k).as_dict() == tuned.as_dict()
     assert _capi.plan(m, n, k).as_dict() == planner.as_dict()          # hfrk_skinny_gemm_plan stays the planner's rule
     assert plan_table.get_plan(m, n, k, packed=True).as_dict() == planner.as_dict()   # another key
-    assert plan_table.get_plan(m + 1, n, k).as_dict() == _capi.plan(m + 1, n, k).as_dict()
+    # the entry also serves the smaller m with the same activation loads (5..8), and no other
+    for mm in (5, 6, 7):
+        assert plan_table.get_plan(mm, n, k).as_dict() == tuned.as_dict(), mm
+    for mm in (4, 9):
+        assert plan_table.get_plan(mm, n, k).as_dict() == _capi.plan(mm, n, k).as_dict(), mm
+    nearer = _capi.GemmPlan(1, 0, 1, 2, 64, planner.panels, planner.slabs, planner.lds_bytes)
+    plan_table.set_plan(6, n, k, nearer)
+    assert plan_table.get_plan(5, n, k).as_dict() == nearer.as_dict()      # the nearest entry at or above m
+    assert plan_table.get_plan(7, n, k).as_dict() == tuned.as_dict()
+    plan_table.remove_plan(6, n, k)
+    # above 16 rows the bucket is a 16-row tile: an entry for 32 serves 17..32
+    big = _capi.plan(32, n, k)
+    big32 = _capi.GemmPlan(big.m_tiles, big.wn, big.wk, big.ch, max(8, big.grid // 2), big.panels, big.slabs, big.lds_bytes)
+    plan_table.set_plan(32, n, k, big32)
+    assert plan_table.get_plan(17, n, k).as_dict() == big32.as_dict()
+    assert plan_table.get_plan(16, n, k).as_dict() == _capi.plan(16, n, k).as_dict()
+    assert plan_table.get_plan(33, n, k).as_dict() == _capi.plan(33, n, k).as_dict()
+    plan_table.remove_plan(32, n, k)
     # a plan that does not fit the shape is refused and changes nothing
     bad = _capi.GemmPlan(1, 0, 1, 1, 128, planner.panels, planner.slabs, planner.lds_bytes)  # 4 rows of activations for m = 8
     with pytest.raises(RuntimeError):
