@@ -29,6 +29,7 @@ const char* hfrk_status_string(int status) {
         case HFRK_BAD_DTYPE: return "unsupported element type";
         case HFRK_HIP_ERROR: return "HIP runtime error (see hfrk_last_hip_error)";
         case HFRK_NOT_INITIALISED: return "workspace not allocated and the stream is capturing: call hfrk_init() first";
+        case HFRK_BAD_FILE: return "plan-table file cannot be read or is not a plan table";
         default: return "unknown status";
     }
 }

@@ -22,6 +22,7 @@ BAD_ALIGNMENT = 8
 BAD_DTYPE = 9
 HIP_ERROR = 10
 NOT_INITIALISED = 11
+BAD_FILE = 12
 
 # enum hfrk_dtype
 F16 = 0
@@ -74,6 +75,7 @@ SIGNATURES = {
     "hfrk_residual_rms_dynamic": (_i, [_p, _p, _p, _f, _p, _p, _p, _i, _i, _i, _i, _p]),
     "hfrk_swiglu_dynamic": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
     "hfrk_quantize_fp8": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
+    "hfrk_plan_table_load": (_i, [ctypes.c_char_p, _i, ctypes.POINTER(_i)]),
 }
 
 _lib = None

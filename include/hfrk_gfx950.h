@@ -35,7 +35,8 @@ enum hfrk_status {
     HFRK_BAD_ALIGNMENT = 8,                 /* a pointer or stride that must be 16-byte aligned is not */
     HFRK_BAD_DTYPE = 9,
     HFRK_HIP_ERROR = 10,                    /* a HIP runtime call failed; hfrk_last_hip_error() has the code */
-    HFRK_NOT_INITIALISED = 11               /* workspace missing and the stream is capturing (call hfrk_init first) */
+    HFRK_NOT_INITIALISED = 11,              /* workspace missing and the stream is capturing (call hfrk_init first) */
+    HFRK_BAD_FILE = 12                      /* a plan-table file that cannot be read or is not a plan table */
 };
 
 /* Element types of 16-bit tensors. */
@@ -111,6 +112,15 @@ int hfrk_skinny_gemm_plan(int m, int n, int k, hfrk_gemm_plan* plan);
 int hfrk_plan_table_set(int m, int n, int k, int packed, const hfrk_gemm_plan* plan);
 int hfrk_plan_table_get(int m, int n, int k, int packed, hfrk_gemm_plan* plan);
 int hfrk_plan_table_clear(void);
+
+/* Install every entry of a plan-table file through hfrk_plan_table_set (host only; `path` is a host string).  The
+ * file is the JSON that this package's grid-search tool writes: {"format": "hfrk-plan-table-1", "entries": [{"m", "n",
+ * "k", "packed", "plan": {"m_tiles", "wn", "wk", "ch", "grid", "panels", "slabs", "lds_bytes"}, ...}]}; other members
+ * are ignored.  strict != 0: the first malformed entry (HFRK_BAD_FILE) or rejected plan (its validation status) ends the
+ * load; strict == 0: such entries are skipped.  *installed (may be NULL) receives the number of entries installed.
+ * Counterpart, for hosts without Python, of shipping the tuned table inside the wrapper
+ * (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102). */
+int hfrk_plan_table_load(const char* path, int strict, int* installed);
 
 /* D[m,n] += scale_tensor[0] * A[m,k] . B[k,n]
  * Replaces `int skinny_gemm(...)` at csrc/op_src/skinny_gemm/skinny_gemm_caller.cu:21-32, the function behind

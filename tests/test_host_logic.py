@@ -405,3 +405,77 @@ def test_every_plan_the_sweep_tool_proposes_is_one_the_library_accepts(m, n, k):
         plan_table.clear()
     assert "workgroup" in families
     assert ("wave-stream" in families) == (m <= 32)
+
+
+def _c_load(path, strict=True):
+    count = ctypes.c_int(-1)
+    status = _capi.load().hfrk_plan_table_load(str(path).encode(), int(strict), ctypes.byref(count))
+    return status, count.value
+
+
+def test_c_loader_installs_the_shipped_table_like_the_python_loader():
+    """hfrk_plan_table_load (for hosts without Python) and plan_table.load read the same file to the same table."""
+    import json
+    from hf_rocm_kernels import plan_table
+    entries = json.load(open(plan_table.DEFAULT_TABLE))["entries"]
+    try:
+        plan_table.clear()
+        assert plan_table.load(plan_table.DEFAULT_TABLE) == len(entries)
+        by_python = [plan_table.get_plan(e["m"], e["n"], e["k"], e["packed"]).as_dict() for e in entries]
+        assert plan_table.clear() == len(entries)
+        assert _c_load(plan_table.DEFAULT_TABLE) == (_capi.SUCCESS, len(entries))
+        by_c = [plan_table.get_plan(e["m"], e["n"], e["k"], e["packed"]).as_dict() for e in entries]
+        assert by_c == by_python == [e["plan"] for e in entries]
+        assert plan_table.clear() == len(entries)
+    finally:
+        plan_table.clear()
+        plan_table.load_from_environment()
+
+
+def test_c_loader_rejects_what_is_not_a_plan_table(tmp_path):
+    import json
+    from hf_rocm_kernels import plan_table
+    good = {"m": 8, "n": 6144, "k": 4096, "packed": False, "plan": _capi.plan(8, 6144, 4096).as_dict(), "us": 7.25, "note": "caf\u00e9 \"x\""}
+    wrong_shape = dict(good, n=100, plan=dict(good["plan"]))        # the plan does not fit n = 100
+    no_grid = dict(good, m=4, plan={k: v for k, v in good["plan"].items() if k != "grid"})
+    fractional = dict(good, m=2, plan=dict(good["plan"], grid=12.5))
+
+    def write(name, text):
+        path = tmp_path / name
+        path.write_text(text)
+        return path
+
+    def table(entries, fmt=plan_table.FORMAT):
+        return json.dumps({"format": fmt, "device": "test", "entries": entries, "extra": [1, {"a": None}, True]}, indent=1)
+
+    try:
+        plan_table.clear()
+        assert _c_load(tmp_path / "missing.json") == (_capi.BAD_FILE, 0)
+        assert _capi.load().hfrk_plan_table_load(None, 1, None) == _capi.BAD_SHAPE
+        for name, text in [("empty.json", ""), ("array.json", "[]"), ("cut.json", table([good])[:-20]), ("trailing.json", table([good]) + "x"),
+                           ("format.json", table([good], fmt="other")), ("noentries.json", json.dumps({"format": plan_table.FORMAT})),
+                           ("deep.json", "[" * 100 + "]" * 100), ("badnum.json", table([good]).replace("6144", "6144."))]:
+            assert _c_load(write(name, text)) == (_capi.BAD_FILE, 0), name
+        assert plan_table.clear() == 0
+        # members the loader does not know are skipped, escapes are read, installed counts entries
+        assert _c_load(write("good.json", table([good]))) == (_capi.SUCCESS, 1)
+        assert plan_table.get_plan(8, 6144, 4096).as_dict() == good["plan"]
+        assert _capi.load().hfrk_plan_table_load(str(tmp_path / "good.json").encode(), 1, None) == _capi.SUCCESS
+        assert plan_table.clear() == 1
+        # strict: the first bad entry ends the load with its status, entries before it stay; lenient: bad entries are skipped
+        mixed = write("mixed.json", table([good, wrong_shape, no_grid, fractional, dict(good, m=7)]))
+        status, count = _c_load(mixed, strict=True)
+        assert status != _capi.SUCCESS and status != _capi.BAD_FILE and count == 1
+        assert plan_table.clear() == 1
+        assert _c_load(write("nogrid.json", table([no_grid])), strict=True) == (_capi.BAD_FILE, 0)
+        assert _c_load(write("frac.json", table([fractional])), strict=True) == (_capi.BAD_FILE, 0)
+        assert _c_load(mixed, strict=False) == (_capi.SUCCESS, 2)
+        assert plan_table.clear() == 2
+        # the file a Python save writes is what the C loader reads
+        saved = tmp_path / "saved.json"
+        plan_table.save([good, dict(good, packed=True)], str(saved))
+        assert _c_load(saved) == (_capi.SUCCESS, 2)
+        assert plan_table.clear() == 2
+    finally:
+        plan_table.clear()
+        plan_table.load_from_environment()
