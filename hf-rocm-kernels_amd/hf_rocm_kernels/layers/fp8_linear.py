@@ -9,7 +9,7 @@ activations and their scales, e.g. from `residual_rms_dynamic` / `swiglu_dynamic
 bias or residual folded into its epilogue.  Larger batches are cut into pieces of 64 rows; a prefill-sized batch
 belongs on a GEMM library and is only handled here so that the layer is always correct.
 """
-from typing import Optional, Tuple, Union
+from typing import Optional, Sequence, Tuple, Union
 
 import torch
 from torch import Tensor
@@ -83,30 +83,79 @@ def apply_fp8_linear(
 
 class Fp8Linear(torch.nn.Module):
     """nn.Linear with an FP8 weight: per-output-channel (default) or per-tensor weight scale, dynamic per-token or
-    static activation scale, optional packed load format.  Inference only."""
+    static activation scale, optional packed load format.  Inference only.
+
+    The tensors are registered buffers (`weight_data`, `weight_scale`, `bias`, `input_scale`), so the layer moves with
+    `.to()` and round-trips through `state_dict()` / `load_state_dict()`; `weight_data` is the (n, k) fp8 weight or,
+    packed, the flat buffer of its PackedWeight (its rank tells which)."""
 
     def __init__(self, weight: Weight, weight_scale: Tensor, bias: Optional[Tensor] = None,
                  input_scale: Optional[Tensor] = None):
         super().__init__()
-        self.weight, self.weight_scale, self.bias, self.input_scale = weight, weight_scale, bias, input_scale
-        self.out_features, self.in_features = (weight.n, weight.k) if isinstance(weight, PackedWeight) else tuple(weight.shape)
+        self.packed = isinstance(weight, PackedWeight)
+        self.out_features, self.in_features = (weight.n, weight.k) if self.packed else tuple(weight.shape)
+        self.register_buffer("weight_data", weight.data if self.packed else weight)
+        self.register_buffer("weight_scale", weight_scale)
+        self.register_buffer("bias", bias)
+        self.register_buffer("input_scale", input_scale)
+        self._refresh()
+        self.register_load_state_dict_post_hook(lambda module, incompatible_keys: module._refresh())
+
+    def _refresh(self) -> None:
+        """The operand handed to the GEMM wrappers: the (n, k) tensor, or a PackedWeight over the current buffer."""
+        self.packed = self.weight_data.dim() == 1
+        self._operand = PackedWeight(self.weight_data, self.out_features, self.in_features) if self.packed else self.weight_data
+
+    def _apply(self, fn, *args, **kwargs):
+        module = super()._apply(fn, *args, **kwargs)
+        self._refresh()
+        return module
+
+    @property
+    def weight(self) -> Weight:
+        return self._operand
 
     @classmethod
     def from_float(cls, linear: torch.nn.Linear, per_channel: bool = True, packed: bool = False,
                    input_scale: Optional[Tensor] = None) -> "Fp8Linear":
-        """Quantise an nn.Linear's weight (scale = amax/448 per output channel or per tensor)."""
+        """Quantise an nn.Linear's weight (scale = amax/448 per output channel or per tensor).  Packing runs on the
+        GPU: `packed=True` needs the layer there."""
         w = linear.weight.detach()
         scale = amax_scale(w, dim=1 if per_channel else None)
         q, _ = fp8_quantize(w, scale)
         weight = pack_weight(q) if packed else q
-        bias = None if linear.bias is None else linear.bias.detach()
+        bias = None if linear.bias is None else linear.bias.detach().clone()
         return cls(weight, scale.reshape(-1).contiguous(), bias, input_scale)
 
     def forward(self, input: Tensor, input_scale: Optional[Tensor] = None, residual: Optional[Tensor] = None) -> Tensor:
         """`input` 16-bit (quantised here) or fp8 with `input_scale`; `residual` is added in the GEMM's epilogue."""
         scale = input_scale if input_scale is not None else self.input_scale
-        return apply_fp8_linear(input, self.weight, self.weight_scale, scale, self.bias, residual)
+        return apply_fp8_linear(input, self._operand, self.weight_scale, scale, self.bias, residual)
 
     def extra_repr(self) -> str:
-        kind = "packed" if isinstance(self.weight, PackedWeight) else "row-major"
+        kind = "packed" if self.packed else "row-major"
         return f"in_features={self.in_features}, out_features={self.out_features}, weight={kind}, bias={self.bias is not None}"
+
+
+def convert_linear_layers(module: torch.nn.Module, per_channel: bool = True, packed: bool = False,
+                          skip: Sequence[str] = ()) -> int:
+    """Replace, in place and recursively, every nn.Linear under `module` that the FP8 GEMM can take (in_features a
+    multiple of 256, 16-bit weight) by an Fp8Linear quantised from it; returns how many were replaced.
+    skip: layers whose dotted name ends with one of these strings stay as they are (e.g. ("lm_head",)).
+    The counterpart, without the serving stack, of switching a model's linear method (reference README.md:95-97)."""
+    replaced = 0
+
+    def visit(parent: torch.nn.Module, prefix: str) -> None:
+        nonlocal replaced
+        for name, child in list(parent.named_children()):
+            full = f"{prefix}.{name}" if prefix else name
+            if isinstance(child, torch.nn.Linear):
+                usable = child.in_features % 256 == 0 and child.weight.dtype in (torch.float16, torch.bfloat16)
+                if usable and not any(full.endswith(suffix) for suffix in skip):
+                    setattr(parent, name, Fp8Linear.from_float(child, per_channel=per_channel, packed=packed))
+                    replaced += 1
+            else:
+                visit(child, full)
+
+    visit(module, "")
+    return replaced

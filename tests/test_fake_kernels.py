@@ -68,3 +68,43 @@ def test_mlp_chain_under_fake_tensors(fused):
                                           _fp8(2 * inter, hidden).t(), one, one, _fp8(hidden, inter).t(), one, one,
                                           add_residual=True, fused=fused)
         assert out.shape == (m, hidden) and out.dtype == torch.bfloat16 and res.shape == (m, hidden)
+
+
+class _Block(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.gate_up = torch.nn.Linear(512, 1024, bias=False)
+        self.down = torch.nn.Linear(512, 512, bias=True)
+        self.odd = torch.nn.Linear(100, 8)        # in_features not a multiple of 256: stays
+        self.lm_head = torch.nn.Linear(512, 64)   # skipped by name
+        self.inner = torch.nn.Sequential(torch.nn.Linear(256, 256), torch.nn.ReLU())
+
+
+def test_convert_linear_layers_and_state_dict_round_trip_on_the_cpu():
+    """Conversion and (de)serialisation are host work: which layers are replaced, what the state dict holds, and that
+    a freshly converted model takes another one's state."""
+    from hf_rocm_kernels.layers import Fp8Linear, convert_linear_layers
+    from oracle import fp8 as ofp8
+    torch.manual_seed(0)
+    model = _Block().to(torch.bfloat16)
+    float_weight = model.down.weight.detach().clone()
+    assert convert_linear_layers(model, skip=("lm_head",)) == 3
+    assert isinstance(model.gate_up, Fp8Linear) and isinstance(model.down, Fp8Linear) and isinstance(model.inner[0], Fp8Linear)
+    assert type(model.odd) is torch.nn.Linear and type(model.lm_head) is torch.nn.Linear
+    assert convert_linear_layers(model) == 1          # a second pass finds only lm_head left
+    # the quantised weight is the oracle's quantisation with per-channel amax/448 scales
+    scale = ofp8.amax_scale(float_weight, dim=1)
+    want, _ = ofp8.fp8_quantize(float_weight, scale)
+    assert torch.equal(model.down.weight_data.view(torch.uint8), want.view(torch.uint8))
+    assert torch.equal(model.down.weight_scale, scale.reshape(-1))
+    state = model.state_dict()
+    assert state["down.weight_data"].dtype == FP8 and state["down.weight_scale"].shape == (512,) and "gate_up.bias" not in state
+    other = _Block().to(torch.bfloat16)
+    convert_linear_layers(other)
+    result = other.load_state_dict(state)
+    assert not result.missing_keys and not result.unexpected_keys
+    for name in ("gate_up", "down", "lm_head"):
+        a, b = getattr(model, name), getattr(other, name)
+        assert torch.equal(a.weight_data.view(torch.uint8), b.weight_data.view(torch.uint8)) and torch.equal(a.weight_scale, b.weight_scale)
+        assert b.weight is b.weight_data and not b.packed
+    assert "weight=row-major" in repr(other.down)

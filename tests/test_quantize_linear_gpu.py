@@ -158,3 +158,45 @@ def test_checked_gemm_operator_raises_where_the_status_operator_returns_a_code()
     assert torch.ops._HFRK_C.skinny_gemm_fused(bad_a, bad_w.t(), d, None, one, None, None, 0, 0) == 3
     with pytest.raises(RuntimeError, match="status 3"):
         torch.ops._HFRK_C.skinny_gemm_checked(bad_a, bad_w.t(), False, 64, d, None, one, None, None, 0, 0)
+
+
+def test_converted_model_tracks_the_float_model_and_reloads_its_state():
+    """convert_linear_layers on a small MLP: outputs track the float model, the state dict (fp8 weights, scales)
+    reloads into a freshly converted model bit for bit, for row-major and packed weights, and a model converted on the
+    CPU works after .to("cuda")."""
+    from hf_rocm_kernels.layers import Fp8Linear, convert_linear_layers
+
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = torch.nn.Linear(1024, 2048, bias=False)
+            self.down = torch.nn.Linear(2048, 1024, bias=True)
+
+        def forward(self, x):
+            return self.down(torch.nn.functional.silu(self.up(x)))
+
+    torch.manual_seed(2)
+    float_model = Mlp().to(torch.bfloat16).cuda()
+    x = torch.randn(6, 1024, device="cuda").to(torch.bfloat16)
+    want = float_model(x).float()
+    for packed in (False, True):
+        model = Mlp().to(torch.bfloat16).cuda()
+        model.load_state_dict(float_model.state_dict())
+        assert convert_linear_layers(model, packed=packed) == 2
+        got = model(x)
+        rel = (got.float() - want).norm() / want.norm()
+        assert rel < 0.08, (packed, float(rel))
+        state = {k: v.clone() for k, v in model.state_dict().items()}
+        assert state["up.weight_data"].dim() == (1 if packed else 2)
+        other = Mlp().to(torch.bfloat16).cuda()
+        convert_linear_layers(other, packed=packed)
+        other.load_state_dict(state)
+        assert torch.equal(other(x), got), packed
+    # converted on the host, moved afterwards: the operand follows the buffer
+    host = Mlp().to(torch.bfloat16)
+    host.load_state_dict({k: v.cpu() for k, v in float_model.state_dict().items()})
+    convert_linear_layers(host)
+    moved = host.to("cuda")
+    assert moved.up.weight.device.type == "cuda" and isinstance(moved.up, Fp8Linear)
+    rel = (moved(x).float() - want).norm() / want.norm()
+    assert rel < 0.08, float(rel)
