@@ -383,11 +383,25 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
                 const int g_last = (int)((hi * (uint32_t)G + (uint32_t)U - 1) / (uint32_t)U) - 1;
 #pragma unroll
                 for (int st = 0; st < ST; ++st) acc[st] = v4f{0.f, 0.f, 0.f, 0.f};
-                for (int gg = g_first; gg <= g_last; ++gg) {
-                    const int sl = (unit_begin(gg, U, G) / S == panel) ? 0 : 1;
+                // kInFlight contributors' shares are requested together (each round trip to memory is paid once per
+                // batch, not once per contributor) and added in id order; past the last one the offset is out of the
+                // buffer's range and the load returns zeros
+                constexpr int kInFlight = ST == 6 ? 1 : ST >= 8 ? 2 : 4;  // what the registers of each variant allow without spilling
+#pragma unroll 1
+                for (int first = g_first; first <= g_last; first += kInFlight) {
+                    v4i share[kInFlight][ST];
 #pragma unroll
-                    for (int st = 0; st < ST; ++st)
-                        acc[st] += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, ws_off(gg, sl, st), 0, kCoherent));
+                    for (int w = 0; w < kInFlight; ++w) {
+                        const int gg = first + w;
+                        const int sl = (unit_begin(gg, U, G) / S == panel) ? 0 : 1;
+#pragma unroll
+                        for (int st = 0; st < ST; ++st)
+                            share[w][st] = __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, gg <= g_last ? ws_off(gg, sl, st) : (int)0x80000000u, 0, kCoherent);
+                    }
+#pragma unroll
+                    for (int w = 0; w < kInFlight; ++w)
+#pragma unroll
+                        for (int st = 0; st < ST; ++st) acc[st] += __builtin_bit_cast(v4f, share[w][st]);
                 }
                 store_panel(panel, flush_par);
             }
