@@ -11,6 +11,8 @@ Cache or from L2.
 Other workloads, same method, for the remaining configurations:
   llama3-70b  M in {1,4,8,16,32} x qkv (10240, 8192), o_proj (8192, 8192), gate_up (57344, 8192), down (8192, 28672)
   scaled-m    M in {16,32,64} x (4096,4096), (28672,4096), (4096,14336) with per-token and per-channel scales
+  llama31-405b-tp8  M in {8,16,32} x o_proj (16384, 2048), qkv (2304, 16384), gate_up (13312, 16384), down (16384, 6656):
+              the shapes the reference tuned for; `--detail` puts the reference's published microseconds beside each case
               (`skinny_gemm_scaled`, activation rows 1 and M-1 drawn 20x larger)
   mlp         the decoder MLP sub-block (`llama_mlp_combined_ops`: residual RMSNorm -> gate_up GEMM -> SwiGLU ->
               down GEMM, output added to the residual), hidden 4096, M in {1, 8, 16}: 3 blocks = 12 launches per step
@@ -60,7 +62,7 @@ WORKLOADS = {
                 "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-8B decode shapes, M=1..16 (us/call in `cases`)",
         "kernel": "hfrk::skinny_gemm_stream_kernel (16 of the 20 launches of a step); with the shipped plan table "
-                  "hfrk::skinny_gemm_kernel<1,8,1,2,1,2> on gate_up at M=8,16 and hfrk::skinny_gemm_ksplit_kernel<1,512> on qkv at M=16",
+                  "hfrk::skinny_gemm_kernel<1,8,1,2,1> on gate_up at M=8,16 and hfrk::skinny_gemm_ksplit_kernel<1,512> on qkv at M=16",
     },
     "llama3-70b": {
         "shapes": [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)],
@@ -79,6 +81,19 @@ WORKLOADS = {
         "metric": "FP8 skinny-GEMM achieved HBM GB/s, per-token x per-channel scales, M=16..64 (us/call in `cases`)",
         "kernel": "hfrk::skinny_gemm_stream_kernel / skinny_gemm_kernel (M=16), hfrk::skinny_gemm_ksplit_kernel (M=32,64 on K=4096), "
                   "hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64 on K=14336 and plan-table entries)",
+    },
+    "llama31-405b-tp8": {
+        "shapes": [("o_proj", 16384, 2048), ("qkv", 2304, 16384), ("gate_up", 13312, 16384), ("down", 16384, 6656)],
+        "ms": [8, 16, 32], "cycle": 7, "scaled": False,
+        "text": "the four weight shapes the reference tuned its kernel for (Llama-3.1-405B shards at tensor-parallel 8, "
+                "hf_rocm_kernels/operators/skinny_gemm/wrapped.py:45-88): M in {8,16,32} x o_proj(16384,2048) qkv(2304,16384) "
+                "gate_up(13312,16384) down(16384,6656); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 12 calls per step",
+        "metric": "FP8 skinny-GEMM achieved HBM GB/s over the reference's tuned shard shapes, M=8..32 (us/call in `cases`)",
+        "kernel": "hfrk::skinny_gemm_stream_kernel / hfrk::skinny_gemm_kernel by plan table",
+        # microseconds the reference's source comments give for its own kernel on these shapes and M buckets
+        # (wrapped.py:49,60,63,66,74,77,82; measured by its authors on MI300X, 5.3 TB/s HBM3)
+        "reference_us": {("o_proj", 8): 11.114, ("qkv", 8): 12.485, ("qkv", 16): 14.301, ("qkv", 32): 17.220,
+                         ("gate_up", 16): 62.136, ("gate_up", 32): 69.251, ("down", 8): 28.668},
     },
 }
 MLP = {"hidden": 4096, "inter": 14336, "ms": [1, 8, 16], "cycle": 12, "eps": 1e-5,
@@ -220,6 +235,10 @@ def time_gemm_cases(torch, spec, call, weights, reps=40):
             rows.append({"shape": name, "n": n, "k": k, "m": m, "us_per_call": round(us, 3), "us_std": round(std, 3),
                          "gbps": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4),
                          "us_cache_hot": round(us_hot, 3)})
+            ref_us = spec.get("reference_us", {}).get((name, m))
+            if ref_us is not None:  # the reference's published time for this case, on its authors' MI300X
+                rows[-1]["reference_us_mi300x"] = ref_us
+                rows[-1]["reference_frac_of_its_peak"] = round(gemm_bytes(m, n, k, 1) / ref_us / 1e3 / 5300.0, 4)
             del cold, hot
     return rows
 
