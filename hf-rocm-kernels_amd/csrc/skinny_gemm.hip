@@ -58,7 +58,10 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* const tbuf_all = lds;
     uint8_t* const act_all = lds + kGemmWaves * RT * kTileBytes;
-    int* const flag = reinterpret_cast<int*>(act_all + 2 * ACT_BYTES);
+    // One word for the "last arriver" verdict of a panel flush.  It lives at the start of wave 0's transposition tile:
+    // during a flush no tile holds weights (the unit's MFMAs are done, the next unit's tiles are written after the flush's
+    // last barrier), and the K-wave reduction that borrows the tiles as scratch writes only those of waves with wk != 0.
+    int* const flag = reinterpret_cast<int*>(tbuf_all);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -495,7 +498,7 @@ static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
 }
 
 constexpr int lds_bytes_for(int mt, int wk, int ch, int rt = 1) {
-    return kGemmWaves * rt * kTileBytes + 2 * 16 * mt * (256 * wk * ch) + 16;
+    return kGemmWaves * rt * kTileBytes + 2 * 16 * mt * (256 * wk * ch);
 }
 
 // m <= 32: every wave streams its own run of (16*RT-row group, 256-byte K chunk) chunks (skinny_gemm_stream.hip).
@@ -580,8 +583,9 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 //   m <= 16          wave-stream kernel (activations per wave from L2: cheap up to 16 rows)
 //   m  > 16          K-split kernel (activations in registers) when one window of it covers k; otherwise the
 //                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
-//                    4 row waves x 2 K waves almost everywhere; 2 x 4 for small weights (more K parallelism where a
-//                    workgroup only gets a few units); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
+//                    4 row waves x 2 K waves almost everywhere; 2 x 4 for narrow weights (n <= 2048: more K parallelism
+//                    where there are few row panels; from 2304 rows on 4 x 2 is 6-15 % faster, measured on 2304..5120 x
+//                    8192..16384 at m = 32, 48); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
@@ -590,7 +594,7 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     const int mt = (m + 15) / 16;
     const double weight_mb = (double)n * k / 1.0e6;
     int first = 4;
-    if (weight_mb < 48.0 && m <= 48) first = 2;
+    if (n <= 2048 && m <= 48) first = 2;
     else if (weight_mb >= 200.0 && m > 48) first = 8;
     const int prefs[3][4] = {{2, 4, 1, 8}, {4, 2, 8, 1}, {8, 4, 2, 1}};
     const int* pref = first == 2 ? prefs[0] : first == 4 ? prefs[1] : prefs[2];

@@ -47,7 +47,7 @@ def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.Gemm
     for wn, ch, rt in itertools.product((1, 2, 4, 8), (1, 2), (1, 2)):  # workgroup: row waves, chunks per slab, tiles per wave
         wk = 8 // wn
         ks = 256 * wk * ch
-        lds = 8 * rt * 4096 + 2 * 16 * mt * ks + 16
+        lds = 8 * rt * 4096 + 2 * 16 * mt * ks
         if k % ks or lds > 160 * 1024 or (rt == 2 and ch != 1):
             continue
         panels, slabs = -(-n // (16 * wn * rt)), k // ks

@@ -76,7 +76,7 @@ def all_plans(m, n, k):
             ks = 256 * wk * ch
             if k % ks:
                 continue
-            lds = 8 * rt * 4096 + 2 * 16 * mt * ks + 16
+            lds = 8 * rt * 4096 + 2 * 16 * mt * ks
             if lds > 160 * 1024:
                 continue
             panels = (n + 16 * wn * rt - 1) // (16 * wn * rt)
@@ -412,7 +412,7 @@ def test_a_plan_table_entry_is_what_a_call_without_a_plan_runs():
     from hf_rocm_kernels.utils.weight_format import pack_weight
     m, n, k = 8, 2048, 4096
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=21)
-    entry = _capi.GemmPlan(1, 2, 4, 1, 23, n // 32, k // 1024, 8 * 4096 + 2 * 16 * 1024 + 16)
+    entry = _capi.GemmPlan(1, 2, 4, 1, 23, n // 32, k // 1024, 8 * 4096 + 2 * 16 * 1024)
     explicit = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     run_ex(a, b, sa, sw, explicit, accumulate=False, plan=entry)
     plan_table.clear()

@@ -348,7 +348,7 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
     assert _capi.load().hfrk_plan_table_set(m, n, 100, 0, ctypes.byref(tuned)) == _capi.BAD_SHAPE
     assert plan_table.get_plan(m, n, k).as_dict() == tuned.as_dict()
     # a workgroup-kernel entry for a shape the planner gives to the wave-stream kernel
-    wg = _capi.GemmPlan(1, 4, 2, 1, 200, n // 64, k // 512, 8 * 4096 + 2 * 16 * 512 + 16)
+    wg = _capi.GemmPlan(1, 4, 2, 1, 200, n // 64, k // 512, 8 * 4096 + 2 * 16 * 512)
     plan_table.set_plan(16, n, k, wg, packed=True)
     path = tmp_path / "table.json"
     plan_table.save([{"m": m, "n": n, "k": k, "packed": False, "plan": tuned.as_dict(), "us": 7.5},
