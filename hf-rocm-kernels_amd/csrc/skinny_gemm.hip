@@ -533,11 +533,12 @@ static int fill_stream_plan(int m, int n, int k, int row_tiles, bool swiglu, int
 static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     const int act_loads = (m + 3) / 4;
     // Two row tiles per chunk halve the activation bytes pulled from L2 per weight byte: needed above 16 rows,
-    // worth it from 9 rows on once a wave's run still has a few 8 KB chunks.
+    // worth it from 9 rows on once a wave's run still has a few 8 KB chunks and a row group has at least 16 of them
+    // (k >= 4096; on 32768 x 2048 at 16 rows one tile per chunk takes 12.9 us, two take 14.5).
     int row_tiles = 1;
     if (act_loads > 4) {
         row_tiles = 2;
-    } else if (act_loads >= 3) {
+    } else if (act_loads >= 3 && k >= 4096) {
         const long chunks2 = (long)((n + 31) / 32) * (k / 256);
         if (chunks2 >= (long)kStreamRt2MinChunksPerWave * kNumCU * kGemmWaves) row_tiles = 2;
     }
