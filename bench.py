@@ -557,7 +557,7 @@ def main():
                    "weight_copies_per_shape": n_copies,
                    "weight_layout": "packed 16x256-byte chunks in MFMA operand order (hfrk_pack_weight)" if args.packed else "row-major [N, K]",
                    "timing": "HIP graph replay, HIP events",
-                   "plan_table": os.environ.get("HFRK_PLAN_TABLE", "shipped (hf_rocm_kernels/plan_tables/gfx950_llama3.json)"),
+                   "plan_table": os.environ.get("HFRK_PLAN_TABLE", "shipped (hf_rocm_kernels/plan_tables/gfx950_*.json)"),
                    "us_per_call_mean": round(ms_per_step * 1e3 / calls, 3), "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),

@@ -512,13 +512,18 @@ static int fill_stream_plan(int m, int n, int k, int row_tiles, bool swiglu, int
     long grid = grid_hint > 0 ? grid_hint : kNumCU;
     if (grid > chunks) grid = chunks;
     if (grid >= 8) grid -= grid % 8;  // whole XCD groups
-    // A grid that divides the row tiles keeps every tile inside one workgroup (no workspace round trip); worth it
-    // when it still fills at least three quarters of the CUs and the runs are short (under 64 chunks per workgroup on the
-    // full grid): on long runs the round trip is small against the CUs left idle (13312 x 16384: 43.6 us on 208
-    // workgroups against 39.7 on 256).
-    if (grid_hint <= 0 && grid == kNumCU && tiles % kNumCU != 0 && chunks < 64L * kNumCU)
-        for (long g = kNumCU - 8; g >= 3 * kNumCU / 4; g -= 8)
-            if (tiles % g == 0) { grid = g; break; }
+    // A grid that divides the row tiles keeps every tile inside one workgroup (no workspace round trip).  Worth the idle
+    // CUs in two cases, both measured: at least three quarters of the CUs and short runs (under 64 chunks per workgroup
+    // on the full grid; 6144 x 4096 on 192), or one or two tiles per workgroup with runs of at most 80 chunks, down to
+    // 160 workgroups (3584 x 18944 on 224: 13.7 against 16.4 us; 5120 x 5120 on 160: 8.0 against 9.0).  On longer runs
+    // the round trip is small against the CUs left idle (13312 x 16384: 43.6 us on 208 against 39.7 on 256).
+    if (grid_hint <= 0 && grid == kNumCU && tiles % kNumCU != 0)
+        for (long g = kNumCU - 8; g >= 5 * kNumCU / 8; g -= 8) {
+            if (tiles % g != 0) continue;
+            const bool short_runs = g >= 3 * kNumCU / 4 && chunks < 64L * kNumCU;
+            const bool few_tiles = tiles / g <= 2 && chunks / g <= 80;
+            if (short_runs || few_tiles) { grid = g; break; }
+        }
     // When every workgroup's share of the weight is a multiple of 512 KB, all workgroups walk addresses that agree in
     // their low 19 bits at the same time and crowd onto a few memory channels (16384 x 8192: 30.5 us on 256 workgroups,
     // 24.8 on 248; 16384 x 16384: 54.3 against 45.8; rows padded by 256 bytes have the same effect).  A grid of 248 breaks

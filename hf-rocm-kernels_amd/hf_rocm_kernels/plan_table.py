@@ -4,10 +4,11 @@ consults in place of its planner's rules.
 Counterpart of the reference's hand-maintained knob table (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102),
 but produced on the box: `benchmarks/skinny_gemm/grid_search.py --save table.json` times every decomposition and
 keeps the winners that beat the planner; `load(path)` installs them through `hfrk_plan_table_set`, which validates
-each plan for its shape.  At import the package installs the table it ships (plan_tables/gfx950_llama3.json) or the
+each plan for its shape.  At import the package installs the tables it ships (plan_tables/gfx950_*.json) or the
 one HFRK_PLAN_TABLE names (`none`: no table).
 """
 import ctypes
+import glob
 import json
 import os
 from typing import Dict, Iterable, List, Optional
@@ -70,17 +71,24 @@ def load(path: str, strict: bool = True) -> int:
     return count
 
 
-DEFAULT_TABLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "plan_tables", "gfx950_llama3.json")
+_TABLE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "plan_tables")
+DEFAULT_TABLE = os.path.join(_TABLE_DIR, "gfx950_llama3.json")   # Llama-3 8B/70B and Llama-3.1-405B TP8 shard shapes
+
+
+def shipped_tables() -> List[str]:
+    """Every table the package ships for this device (plan_tables/gfx950_*.json), in name order."""
+    return sorted(glob.glob(os.path.join(_TABLE_DIR, "gfx950_*.json")))
 
 
 def load_from_environment() -> Optional[int]:
     """Called when the package is imported.  HFRK_PLAN_TABLE=<file> installs that table, HFRK_PLAN_TABLE=none
-    installs nothing, unset installs the table shipped with the package (entries tuned on an MI355X for the
-    Llama-3 8B/70B projection shapes, the way the reference ships its tuned shapes inside its wrapper).  Non-strict:
+    installs nothing, unset installs the tables shipped with the package (plan_tables/gfx950_*.json: entries tuned on an
+    MI355X for the projection shapes of common models, the way the reference ships its tuned shapes inside its wrapper).  Non-strict:
     entries this library version rejects are skipped."""
     path = os.environ.get(ENV_VAR)
     if path is None:
-        path = DEFAULT_TABLE if os.path.exists(DEFAULT_TABLE) else ""
+        tables = shipped_tables()
+        return sum(load(t, strict=False) for t in tables) if tables else None
     if not path or path.lower() == "none":
         return None
     return load(path, strict=False)

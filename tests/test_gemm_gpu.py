@@ -433,3 +433,40 @@ def test_a_plan_table_entry_is_what_a_call_without_a_plan_runs():
     assert torch.equal(six, explicit[:6])
     check_against_oracle(after, a, b, sa, sw)
     check_against_oracle(before, a, b, sa, sw)
+
+
+def _shipped_entries():
+    import json
+    from hf_rocm_kernels import plan_table
+    entries = []
+    for path in plan_table.shipped_tables():
+        for e in json.load(open(path))["entries"]:
+            entries.append(pytest.param(e, id=f"{e['m']}x{e['n']}x{e['k']}{'p' if e['packed'] else ''}"))
+    return entries
+
+
+@pytest.mark.parametrize("entry", _shipped_entries())
+def test_every_shipped_plan_table_entry_computes_what_the_planner_s_plan_computes(entry):
+    """Each tuned entry is another decomposition of the same product: a call that picks it up from the table must agree
+    with the same call run on the planner's plan (itself checked against the oracle above) to within the reassociation
+    of fp32 sums, on the entry's own full-size shape and weight layout."""
+    from hf_rocm_kernels import _capi, plan_table, skinny_gemm_scaled
+    from hf_rocm_kernels.utils.weight_format import pack_weight
+    m, n, k, packed = entry["m"], entry["n"], entry["k"], entry["packed"]
+    assert plan_table.get_plan(m, n, k, packed).as_dict() == entry["plan"], "the shipped table is not installed"
+    g = torch.Generator(device="cuda").manual_seed(m + n + k)
+    def codes(rows, cols):  # finite e4m3fn codes of both signs
+        c = torch.randint(0, 120, (rows, cols), generator=g, device="cuda", dtype=torch.uint8)
+        sign = torch.randint(0, 2, (rows, cols), generator=g, device="cuda", dtype=torch.uint8) << 7
+        return (c | sign).view(torch.float8_e4m3fn)
+    a, w = codes(m, k), codes(n, k)
+    sa = torch.full((1,), 2.0 ** -8, device="cuda")
+    sw = torch.full((1,), 2.0 ** -8, device="cuda")
+    want = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    run_ex(a, w.t(), sa, sw, want, accumulate=False, plan=_capi.plan(m, n, k))
+    got = skinny_gemm_scaled(a, pack_weight(w) if packed else w.t(), sa, sw)
+    torch.cuda.synchronize()
+    err = (got.float() - want.float()).abs()
+    bound = want.float().abs() * 2.0 ** -7 + 2.0 ** -6   # one bf16 step of the result, plus the cancellation floor
+    assert bool((err <= bound).all()), float((err - bound).max())
+    assert float(want.float().abs().mean()) > 0.1

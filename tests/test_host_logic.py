@@ -369,7 +369,9 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
     monkeypatch.delenv(plan_table.ENV_VAR)
     shipped = plan_table.load_from_environment()   # the table shipped with the package: every entry must be accepted
     import json
-    assert shipped == len(json.load(open(plan_table.DEFAULT_TABLE))["entries"]) and shipped > 0
+    tables = plan_table.shipped_tables()
+    assert plan_table.DEFAULT_TABLE in tables and len(tables) >= 2
+    assert shipped == sum(len(json.load(open(t))["entries"]) for t in tables) and shipped > 0
     assert plan_table.clear() == shipped
     other = tmp_path / "other.json"
     other.write_text('{"format": "something else", "entries": []}')
