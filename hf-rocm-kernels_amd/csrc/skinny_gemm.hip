@@ -598,9 +598,31 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 //                    4 row waves x 2 K waves almost everywhere; 2 x 4 for narrow weights (n <= 2048: more K parallelism
 //                    where there are few row panels; from 2304 rows on 4 x 2 is 6-15 % faster, measured on 2304..5120 x
 //                    8192..16384 at m = 32, 48); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
+// workgroup decomposition with wn row waves x (8 / wn) K waves and ch chunks per slab, on min(256, units) workgroups
+static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_plan* plan) {
+    const int mt = (m + 15) / 16, wk = kGemmWaves / wn, ks = 256 * wk * ch;
+    if (k % ks != 0 || lds_bytes_for(mt, wk, ch) > kLdsLimit) return HFRK_INVALID_CONFIG;
+    const long panels = (n + 16 * wn - 1) / (16 * wn);
+    if (panels > kMaxPanels) return HFRK_BAD_SHAPE;
+    const long units = panels * (k / ks);
+    plan->m_tiles = mt;
+    plan->wn = wn;
+    plan->wk = wk;
+    plan->ch = ch;
+    plan->grid = (int)(units < kNumCU ? units : kNumCU);
+    plan->panels = (int)panels;
+    plan->slabs = k / ks;
+    plan->lds_bytes = lds_bytes_for(mt, wk, ch);
+    return HFRK_SUCCESS;
+}
+
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    // k = 1024 is four chunks per row tile: too few for the wave-stream split and half a K-split window.  Four K waves
+    // cover it in one slab, so nothing is exchanged between workgroups (1024 x 1024: 4.2 against 5.2 us at 1 row,
+    // 5120 x 1024: 5.7 against 7.3 at 32 rows); on weights wider than 12288 rows the other kernels catch up.
+    if (k == 1024 && n <= 12288 && fill_workgroup_plan(m, n, k, 2, 1, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (m <= 16) {
         // Small weights: with at most one 4 KB chunk per wave the wave-stream split leaves waves idle and sends every row
         // tile through the workspace; one workgroup per tile, its 8 waves splitting K, finishes inside the workgroup
@@ -610,34 +632,15 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         return make_stream_plan(m, n, k, plan);
     }
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
-    const int mt = (m + 15) / 16;
     const double weight_mb = (double)n * k / 1.0e6;
     int first = 4;
     if (n <= 2048 && m <= 48) first = 2;
     else if (weight_mb >= 200.0 && m > 48) first = 8;
     const int prefs[3][4] = {{2, 4, 1, 8}, {4, 2, 8, 1}, {8, 4, 2, 1}};
     const int* pref = first == 2 ? prefs[0] : first == 4 ? prefs[1] : prefs[2];
-    for (int pi = 0; pi < 4; ++pi) {
-        const int wn = pref[pi], wk = kGemmWaves / wn;
-        for (int ch = 1; ch <= 2; ++ch) {
-            const int ks = 256 * wk * ch;
-            if (k % ks != 0) continue;
-            if (lds_bytes_for(mt, wk, ch) > kLdsLimit) continue;
-            const int bn = 16 * wn;
-            const long panels = (n + bn - 1) / bn;
-            if (panels > kMaxPanels) continue;
-            const long units = panels * (k / ks);
-            plan->m_tiles = mt;
-            plan->wn = wn;
-            plan->wk = wk;
-            plan->ch = ch;
-            plan->grid = (int)(units < kNumCU ? units : kNumCU);
-            plan->panels = (int)panels;
-            plan->slabs = k / ks;
-            plan->lds_bytes = lds_bytes_for(mt, wk, ch);
-            return HFRK_SUCCESS;
-        }
-    }
+    for (int pi = 0; pi < 4; ++pi)
+        for (int ch = 1; ch <= 2; ++ch)
+            if (fill_workgroup_plan(m, n, k, pref[pi], ch, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     return HFRK_BAD_SHAPE;
 }
 
