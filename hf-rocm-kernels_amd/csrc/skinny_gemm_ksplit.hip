@@ -181,6 +181,44 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
         }
     };
 
+    // Several windows (S > 1): a unit's share of its tile goes to the workspace and an arrival counter decides who adds
+    // the shares.  Store, acknowledgement, counter round trip and the verdict are spread over two units so that none of
+    // them is waited for where it was issued: the share is stored at the end of unit i, acknowledged and counted at the
+    // top of unit i+1 (when nothing else of this wave is in flight), and the counter's answer is looked at after unit
+    // i+1's MFMAs; only then does the last arriver add the shares and store the tile.
+    // (The 1 KB-per-wave variants have no register to carry this state across units: they count and settle on the spot.)
+    constexpr bool kDeferred = KW < 1024;
+    int stored_tile = -1;   // share in flight, arrival not yet counted
+    int counted_tile = -1;  // arrival counted, answer not yet looked at
+    int ticket = 0;         // lane 0: what the counter held before this wave's arrival
+    auto count_arrival = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's share acknowledged before the arrival is counted
+        if (lane == 0) ticket = atomicAdd(a.counters + stored_tile * MT + wv, 1);
+        counted_tile = stored_tile;
+        stored_tile = -1;
+    };
+    auto settle = [&]() __attribute__((always_inline)) {
+        const int t = counted_tile;
+        counted_tile = -1;
+        int last = 0;
+        if (lane == 0) {
+            last = ticket == S - 1;
+            if (last) a.counters[t * MT + wv] = 0;  // ready for the next launch
+        }
+        if (__builtin_amdgcn_readfirstlane(last) == 0) return;
+        v4f total = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+        for (int j0 = 0; j0 < S; j0 += 4) {
+            v4i q[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)  // four shares in flight; past the last window the load is out of range: zeros
+                q[x] = __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, j0 + x < S ? ((((j0 + x) * T + t) * MT + wv) * 64 + lane) * 16 : (int)kOutOfRange, 0, kCoherent);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) total += __builtin_bit_cast(v4f, q[x]);
+        }
+        epilogue(t, wv, total);
+    };
+
     // ---- unit loop ----------------------------------------------------------------------------------------------------
 #pragma unroll 1
     for (int i = 0; i < count; ++i) {
@@ -189,6 +227,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
             for (int c = 0; c < KCH; ++c)
 #pragma unroll
                 for (int t = 0; t < 4; ++t) *reinterpret_cast<v4i*>(tw + c * kTileBytes + wr_off[t]) = wq[c][t];
+        }
+        if constexpr (kDeferred) {
+            if (S > 1 && wv < MT && stored_tile >= 0) count_arrival();
         }
         const bool more = i + 1 < count;
         bool new_window = false;
@@ -246,33 +287,21 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
             v4f sum = part[0];
 #pragma unroll
             for (int w = 1; w < kGemmWaves; ++w) sum += part[w];
-            bool finish = true;
             if (S > 1) {
+                if constexpr (kDeferred) {
+                    if (counted_tile >= 0) settle();  // the unit before this one
+                }
                 // this window's share of tile (tile, wv) goes to the workspace; whoever completes the tile adds the shares
                 const int slot = (win * T + tile) * MT + wv;
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, sum), ws_rsrc, (slot * 64 + lane) * 16, 0, kCoherent);
-                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every lane's store acknowledged before the arrival is counted
-                int last = 0;
-                if (lane == 0) {
-                    int* const counter = a.counters + tile * MT + wv;
-                    last = atomicAdd(counter, 1) == S - 1;
-                    if (last) *counter = 0;  // ready for the next launch
+                stored_tile = tile;
+                if constexpr (!kDeferred) {
+                    count_arrival();
+                    settle();
                 }
-                finish = __builtin_amdgcn_readfirstlane(last) != 0;
-                if (finish) {
-                    sum = v4f{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-                    for (int j0 = 0; j0 < S; j0 += 4) {
-                        v4i q[4];
-#pragma unroll
-                        for (int x = 0; x < 4; ++x)  // four shares in flight; past the last window the load is out of range: zeros
-                            q[x] = __builtin_amdgcn_raw_buffer_load_b128(ws_rsrc, j0 + x < S ? ((((j0 + x) * T + tile) * MT + wv) * 64 + lane) * 16 : (int)kOutOfRange, 0, kCoherent);
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) sum += __builtin_bit_cast(v4f, q[x]);
-                    }
-                }
+            } else {
+                epilogue(tile, wv, sum);
             }
-            if (finish) epilogue(tile, wv, sum);
         }
         // advance to the unit whose weights are already on their way
         if (more) {
@@ -281,6 +310,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
                 win = iwin;
                 load_window(win);
             }
+        }
+    }
+    if constexpr (kDeferred) {
+        if (S > 1 && wv < MT) {  // the last unit's share
+            if (stored_tile >= 0) count_arrival();
+            if (counted_tile >= 0) settle();
         }
     }
 }
