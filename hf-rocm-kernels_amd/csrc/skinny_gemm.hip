@@ -26,9 +26,12 @@
 //    every slab of the panel it writes D directly, otherwise it parks its fp32 partial in the workspace and the
 //    workgroup that arrives last (per-panel counter) adds the partials in workgroup order -- a fixed order, so
 //    results are bit-reproducible -- applies the scales once, adds D (accumulate mode) and rounds once.
+#include <functional>
 #include <mutex>
+#include <thread>
 #include <type_traits>
 #include <unordered_map>
+#include <vector>
 
 #include "skinny_gemm_args.h"
 
@@ -331,7 +334,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
     // fp32 partial of (workgroup gg, slot): [wn][rt * MT + mt][lane] float4.  Partials cross XCDs, whose L2s are not coherent
     // with each other: they are written through to memory and read past the caches (sc0 sc1 on both sides), which
     // keeps them coherent per location without the L2 write-back / invalidate a device-scope fence would cost.
-    const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
+    const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, a.ws_bytes);
     auto ws_off = [&](int gg, int slot, int st) __attribute__((always_inline)) -> int {
         return (((gg * 2 + slot) * (WN * ST) + wn * ST + st) * 64 + lane) * 16;
     };
@@ -456,44 +459,83 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_kernel(const GemmArg
 // ------------------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------------------
-struct DeviceState {
+// Split-K workspaces.  Partial sums that cross workgroups and the arrival counters that decide who adds them live in a
+// workspace; two GEMMs that run at the same time must not share one, so every stream gets its own from a small per-device
+// pool (launches on one stream are ordered, so they can share).  The reference needs none of this: it adds fp16 atomics
+// into the caller's output (consumers/mfma_16x16x32_consumer.cu:155-163), which makes its calls independent of each other.
+struct Workspace {
     float* ws = nullptr;
     int* counters = nullptr;
 };
-static DeviceState g_dev[64];
+struct DeviceState {
+    std::vector<Workspace> pool;                 // allocated workspaces
+    std::vector<int> unassigned;                 // indices into pool that no stream owns
+    std::unordered_map<uint64_t, int> by_stream; // stream key -> index into pool
+};
+static DeviceState g_dev[kMaxDevices];
 static std::mutex g_mutex;
 
-static int ensure_workspace(int dev, hipStream_t stream, DeviceState** out) {
-    if (dev < 0 || dev >= 64) return HFRK_BAD_SHAPE;
-    {
-        std::lock_guard<std::mutex> lock(g_mutex);
-        if (g_dev[dev].ws != nullptr) {
-            *out = &g_dev[dev];
-            return HFRK_SUCCESS;
-        }
+constexpr int kInitialWorkspaces = 4;  // allocated by hfrk_init: the streams a capture may meet for the first time
+constexpr int kMaxWorkspaces = 64;     // 68 MB each; a 65th concurrent stream gets HFRK_NO_WORKSPACE
+
+__global__ void zero_ints_kernel(int* p, int count) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) p[i] = 0;
+}
+
+// The per-thread default stream is one handle for as many streams as there are threads.
+static uint64_t stream_key(hipStream_t stream) {
+    uint64_t key = reinterpret_cast<uintptr_t>(stream);
+    if (stream == hipStreamPerThread) key ^= (uint64_t)std::hash<std::thread::id>()(std::this_thread::get_id()) << 8;
+    return key;
+}
+
+// caller holds g_mutex
+static int grow_pool(DeviceState& d) {
+    Workspace w;
+    HFRK_HIP_TRY(hipMalloc(&w.ws, kWsFloats * sizeof(float)));
+    hipError_t e = hipMalloc(&w.counters, kMaxPanels * sizeof(int));
+    if (e == hipSuccess) e = hipMemset(w.counters, 0, kMaxPanels * sizeof(int));
+    if (e != hipSuccess) {
+        (void)hipFree(w.ws);
+        if (w.counters) (void)hipFree(w.counters);
+        set_last_hip_error(e);
+        return HFRK_HIP_ERROR;
     }
-    if (stream != nullptr) {
-        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
-            return HFRK_NOT_INITIALISED;
-    }
+    d.pool.push_back(w);
+    d.unassigned.push_back((int)d.pool.size() - 1);
+    return HFRK_SUCCESS;
+}
+
+static bool is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+// The workspace of `stream` on device `dev`: the one it already owns, else an unassigned one, else (outside a capture)
+// a newly allocated one.
+static int workspace_for(int dev, hipStream_t stream, Workspace* out) {
+    if (dev < 0 || dev >= kMaxDevices) return HFRK_BAD_SHAPE;
+    DeviceState& d = g_dev[dev];
+    const uint64_t key = stream_key(stream);
     std::lock_guard<std::mutex> lock(g_mutex);
-    if (g_dev[dev].ws == nullptr) {
-        float* ws = nullptr;
-        int* counters = nullptr;
-        HFRK_HIP_TRY(hipMalloc(&ws, kWsFloats * sizeof(float)));
-        hipError_t e = hipMalloc(&counters, kMaxPanels * sizeof(int));
-        if (e == hipSuccess) e = hipMemset(counters, 0, kMaxPanels * sizeof(int));
-        if (e != hipSuccess) {
-            (void)hipFree(ws);
-            if (counters) (void)hipFree(counters);
-            set_last_hip_error(e);
-            return HFRK_HIP_ERROR;
-        }
-        g_dev[dev].counters = counters;
-        g_dev[dev].ws = ws;
+    const auto it = d.by_stream.find(key);
+    if (it != d.by_stream.end()) {
+        *out = d.pool[it->second];
+        return HFRK_SUCCESS;
     }
-    *out = &g_dev[dev];
+    if (d.unassigned.empty()) {
+        if (is_capturing(stream)) return HFRK_NOT_INITIALISED;
+        if ((int)d.pool.size() >= kMaxWorkspaces) return HFRK_NO_WORKSPACE;
+        do {  // the first launch on a device does what hfrk_init does
+            const int rc = grow_pool(d);
+            if (rc != HFRK_SUCCESS) return rc;
+        } while ((int)d.pool.size() < kInitialWorkspaces);
+    }
+    const int idx = d.unassigned.back();
+    d.unassigned.pop_back();
+    d.by_stream.emplace(key, idx);
+    *out = d.pool[idx];
     return HFRK_SUCCESS;
 }
 
@@ -794,8 +836,8 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
 
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
-    DeviceState* st = nullptr;
-    const int rc = ensure_workspace(dev, stream, &st);
+    Workspace st;
+    const int rc = workspace_for(dev, stream, &st);
     if (rc != HFRK_SUCCESS) return rc;
 
     GemmArgs args;
@@ -820,8 +862,9 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.grid = p.grid;
     args.chunks_q = args.units / p.grid;
     args.chunks_r = args.units % p.grid;
-    args.ws = st->ws;
-    args.counters = st->counters;
+    args.ws = st.ws;
+    args.ws_bytes = (uint32_t)(kWsFloats * sizeof(float));
+    args.counters = st.counters;
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, p.lds_bytes, stream);
     switch (p.m_tiles) {
@@ -840,8 +883,49 @@ extern "C" {
 int hfrk_init(void) {
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
-    hfrk::DeviceState* st = nullptr;
-    return hfrk::ensure_workspace(dev, nullptr, &st);
+    if (dev < 0 || dev >= hfrk::kMaxDevices) return HFRK_BAD_SHAPE;
+    std::lock_guard<std::mutex> lock(hfrk::g_mutex);
+    hfrk::DeviceState& d = hfrk::g_dev[dev];
+    while ((int)d.pool.size() < hfrk::kInitialWorkspaces) {
+        const int rc = hfrk::grow_pool(d);
+        if (rc != HFRK_SUCCESS) return rc;
+    }
+    return HFRK_SUCCESS;
+}
+
+int hfrk_release_stream(void* stream) {
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= hfrk::kMaxDevices) return HFRK_BAD_SHAPE;
+    std::lock_guard<std::mutex> lock(hfrk::g_mutex);
+    hfrk::DeviceState& d = hfrk::g_dev[dev];
+    const auto it = d.by_stream.find(hfrk::stream_key(static_cast<hipStream_t>(stream)));
+    if (it == d.by_stream.end()) return HFRK_SUCCESS;
+    d.unassigned.push_back(it->second);
+    d.by_stream.erase(it);
+    return HFRK_SUCCESS;
+}
+
+int hfrk_reset_workspace(void* stream) {
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= hfrk::kMaxDevices) return HFRK_BAD_SHAPE;
+    std::lock_guard<std::mutex> lock(hfrk::g_mutex);
+    for (const hfrk::Workspace& w : hfrk::g_dev[dev].pool) {
+        hipLaunchKernelGGL(hfrk::zero_ints_kernel, dim3(hfrk::kMaxPanels / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           w.counters, hfrk::kMaxPanels);
+        HFRK_HIP_TRY(hipGetLastError());
+    }
+    return HFRK_SUCCESS;
+}
+
+int hfrk_workspace_id(void* stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= hfrk::kMaxDevices) return -1;
+    std::lock_guard<std::mutex> lock(hfrk::g_mutex);
+    const hfrk::DeviceState& d = hfrk::g_dev[dev];
+    const auto it = d.by_stream.find(hfrk::stream_key(static_cast<hipStream_t>(stream)));
+    return it == d.by_stream.end() ? -1 : it->second;
 }
 
 int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, int A_producers, int B_producers,

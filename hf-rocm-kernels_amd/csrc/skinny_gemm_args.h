@@ -10,6 +10,7 @@ constexpr int kGemmThreads = kGemmWaves * kWave;
 constexpr int kTileBytes = 4096;       // 16 rows x 256 B: one K chunk of one 16-row tile
 constexpr int kLdsLimit = 160 * 1024;  // LDS per CU on gfx950
 constexpr int kMaxPanels = 1 << 20;    // arrival counters (one per row panel / row tile)
+constexpr int kMaxDevices = 64;     // devices this library keeps per-device state for
 constexpr int kMaxGrid = 4 * kNumCU;   // persistent workgroups: up to 4 per CU when LDS and registers allow
 constexpr size_t kWsFloats = (size_t)2 * kMaxGrid * kGemmWaves * 4 * 256;  // 2 slots x grid x up to 32 KB of fp32 partials
 
@@ -27,8 +28,9 @@ struct GemmArgs {
     int d_dtype;             // dtype of D; with the SwiGLU epilogue the 16-bit dtype the projections are rounded to
     int panels, slabs, units, grid;  // units = panels * slabs
     int chunks_q, chunks_r;  // stream kernel: (panels * slabs) / grid and % grid
-    float* ws;
-    int* counters;
+    float* ws;               // fp32 partial sums that cross workgroups
+    uint32_t ws_bytes;       // size of ws: accesses beyond it are dropped by the buffer range check
+    int* counters;           // arrival counters, zero between launches
 };
 
 // wave-stream kernel (m <= 32), skinny_gemm_stream.hip: act_loads = ceil(m/4) 16-byte activation loads per lane and

@@ -107,7 +107,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     __builtin_amdgcn_sched_barrier(0);  // keep the set-up below behind the first request
 
     // ---- the rest of the set-up -----------------------------------------------------------------------------------
-    const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, (uint32_t)(kWsFloats * sizeof(float)));
+    const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, a.ws_bytes);
     const int n_out = SWIGLU ? (a.n >> 1) : a.n;  // columns of D
     const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)n_out * (SWIGLU ? 1u : 2u));
     const __amdgpu_buffer_rsrc_t base_rsrc = make_rsrc(a.base, a.base ? (uint32_t)a.m * (uint32_t)a.n * 2u : 0u);

@@ -23,6 +23,7 @@ BAD_DTYPE = 9
 HIP_ERROR = 10
 NOT_INITIALISED = 11
 BAD_FILE = 12
+NO_WORKSPACE = 13
 
 # enum hfrk_dtype
 F16 = 0
@@ -55,6 +56,9 @@ _i, _p, _f = ctypes.c_int, ctypes.c_void_p, ctypes.c_float
 SIGNATURES = {
     "hfrk_version": (_i, []),
     "hfrk_init": (_i, []),
+    "hfrk_release_stream": (_i, [_p]),
+    "hfrk_reset_workspace": (_i, [_p]),
+    "hfrk_workspace_id": (_i, [_p]),
     "hfrk_last_hip_error": (_i, []),
     "hfrk_status_string": (ctypes.c_char_p, [_i]),
     "hfrk_skinny_gemm_validate": (_i, [_i] * 13),

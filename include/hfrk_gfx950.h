@@ -3,8 +3,9 @@
  *
  * Plain pointers and sizes only; every pointer is a DEVICE pointer unless stated otherwise, every call is
  * asynchronous on `stream` (a hipStream_t passed as void*; NULL = the default stream) and launches on the
- * device that is current on the calling thread.  No call synchronises, reads back, or (after hfrk_init for
- * that device) allocates, so all of them can be recorded into a HIP graph.
+ * device that is current on the calling thread.  No call synchronises or reads back, and after hfrk_init for that
+ * device none allocates (unless more than four streams launch GEMMs, see hfrk_init), so all of them can be recorded
+ * into a HIP graph.
  *
  * FP8 is OCP e4m3fn (bias 7, max 448, no infinities) -- the format gfx950's matrix cores implement.  The
  * reference was written for gfx942's e4m3fnuz; on the same bits an fnuz value is half the fn value.
@@ -36,7 +37,8 @@ enum hfrk_status {
     HFRK_BAD_DTYPE = 9,
     HFRK_HIP_ERROR = 10,                    /* a HIP runtime call failed; hfrk_last_hip_error() has the code */
     HFRK_NOT_INITIALISED = 11,              /* workspace missing and the stream is capturing (call hfrk_init first) */
-    HFRK_BAD_FILE = 12                      /* a plan-table file that cannot be read or is not a plan table */
+    HFRK_BAD_FILE = 12,                     /* a plan-table file that cannot be read or is not a plan table */
+    HFRK_NO_WORKSPACE = 13                  /* more streams hold a split-K workspace than the library allows (hfrk_release_stream) */
 };
 
 /* Element types of 16-bit tensors. */
@@ -76,12 +78,28 @@ typedef struct hfrk_gemm_plan {
 /* Library version, for the binding to check. */
 int hfrk_version(void);
 
-/* Allocate (once per device) the split-K workspace of the current device.  Idempotent, thread-safe.
- * Must have run on a device before a GEMM on that device is captured into a graph.  All GEMM launches on one
- * device share this workspace and its arrival counters: order them on one stream (or one chain of graph nodes);
- * two GEMMs running at the same time on one device would mix their partial sums.  No reference counterpart
- * (the reference accumulates with fp16 atomics into a caller-zeroed output instead of using a workspace). */
+/* Split-K workspaces.  A GEMM whose row tiles are shared between workgroups parks fp32 partial sums in a workspace
+ * (64 MB + 4 MB of arrival counters) and the last workgroup to arrive adds them.  Two GEMMs that run at the same time
+ * must not share a workspace, so each stream that launches a GEMM owns one, taken from a per-device pool on the
+ * stream's first launch and kept from then on; launches on different streams are therefore independent of each other,
+ * as the reference's are (it needs no workspace: it adds fp16 atomics into the caller's zeroed output,
+ * csrc/op_src/skinny_gemm/consumers/mfma_16x16x32_consumer.cu:155-163).
+ *   hfrk_init             allocates the first 4 workspaces of the current device.  Idempotent, thread-safe.  The pool
+ *                         grows by itself (up to 64) when a fifth stream appears, except while that stream is being
+ *                         captured into a graph (no allocation inside a capture): then the call returns
+ *                         HFRK_NOT_INITIALISED, so run hfrk_init, and one launch per further stream, before capturing.
+ *   hfrk_release_stream   returns the stream's workspace to the pool (before destroying a stream that has launched
+ *                         GEMMs; the stream must have finished them).  HFRK_SUCCESS also when it owned none.
+ *   hfrk_reset_workspace  zeroes the arrival counters of every workspace of the current device, asynchronously on
+ *                         `stream`: for after a launch that did not run to its end (a device fault, a killed process
+ *                         sharing the context).  No GEMM may be running on the device meanwhile.
+ *   hfrk_workspace_id     index of the workspace `stream` owns on the current device, or -1 (diagnostics and tests).
+ * A graph records the workspace of the stream it was captured on: replay it ordered with that stream's other GEMM work,
+ * or capture on a stream of its own, as torch.cuda.graph does. */
 int hfrk_init(void);
+int hfrk_release_stream(void* stream);
+int hfrk_reset_workspace(void* stream);
+int hfrk_workspace_id(void* stream);
 
 /* hipError_t of the last failed HIP call on this thread (0 if none). */
 int hfrk_last_hip_error(void);

@@ -470,3 +470,187 @@ def test_every_shipped_plan_table_entry_computes_what_the_planner_s_plan_compute
     bound = want.float().abs() * 2.0 ** -7 + 2.0 ** -6   # one bf16 step of the result, plus the cancellation floor
     assert bool((err <= bound).all()), float((err - bound).max())
     assert float(want.float().abs().mean()) > 0.1
+
+
+# ---- BASELINE config 3 (Llama-3-70B, unsharded) at full size against the oracle ------------------------------------------
+
+def _check_columns_against_oracle(cases, b_codes_nk, sw, cols=4096):
+    """cases: [(label, out [m,n] on the device, a [m,k] fp8 on the host, sa [1 or m] on the host)].  The oracle's two
+    checks of `check_against_oracle` (rtol/atol 1e-2 against the fp32 path; 1 ulp + 2^-16 sum|a b| against the exact
+    product), evaluated one slice of output columns at a time so that the float64 copy of a 470 MB weight is never
+    held whole, and with each slice decoded once for all the cases that share the weight."""
+    og = _oracle()
+    from oracle import fp8 as ofp8
+    n = b_codes_nk.shape[0]
+    outs = [(label, out.cpu(), a, sa) for label, out, a, sa in cases]
+    for c0 in range(0, n, cols):
+        c1 = min(n, c0 + cols)
+        w64 = torch.from_numpy(ofp8.decode(b_codes_nk[c0:c1].view(torch.uint8)))   # [cols, k] float64
+        w64_abs = w64.abs()
+        w32 = w64.float()
+        swc = sw if sw.numel() == 1 else sw[c0:c1]
+        for label, got, a, sa in outs:
+            a64 = torch.from_numpy(ofp8.decode(a.view(torch.uint8)))
+            scale = sa.double().reshape(-1, 1) * swc.double().reshape(1, -1)
+            exact = (a64 @ w64.t()) * scale
+            bound = og.ulp16(exact, got.dtype) + (a64.abs() @ w64_abs.t()) * scale.abs() * 2.0 ** -16
+            g = got[:, c0:c1]
+            assert not g.isnan().any(), label
+            worst = ((g.double() - exact).abs() / bound).max().item()
+            assert worst <= 1.0, f"{label}, columns {c0}..{c1}: error is {worst} x the bound from the exact product"
+            ref32 = ((a64.float() * sa.float().reshape(-1, 1)) @ (w32 * swc.float().reshape(-1, 1)).t()).to(got.dtype).float()
+            err = (g.float() - ref32).abs()
+            tol = 1e-2 + 1e-2 * ref32.abs()
+            assert (err <= tol).all(), f"{label}, columns {c0}..{c1}: excess over rtol/atol 1e-2: {(err - tol).max().item()}"
+
+
+@pytest.mark.parametrize("name,n,k", [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192),
+                                      ("down", 8192, 28672)])
+def test_llama3_70b_shapes_match_the_oracle(name, n, k):
+    """Every (N, K) of BASELINE's Llama-3-70B configuration, row-major at M = 1, 8, 32 and from the packed weight at
+    M = 8, through the operator (so with the plan the installed table or the planner gives the shape), against the
+    exact oracle at full size."""
+    from hf_rocm_kernels import plan_table, skinny_gemm, skinny_gemm_scaled
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    from hf_rocm_kernels.utils.weight_format import pack_weight
+    _, b, _, sw = generate_llama_gemm_data(1, n, k, seed=70 + n % 7, device="cpu")
+    b_dev = b.t().contiguous().cuda().t()      # [k, n] view of the [n, k] weight
+    sw_dev = sw.cuda()
+    cases = []
+    for m in (1, 8, 32):
+        a, _, sa, _ = generate_llama_gemm_data(m, 16, k, seed=700 + m, device="cpu")
+        print(f"{name} m={m}: plan {plan_table.get_plan(m, n, k).as_dict()}", flush=True)
+        out = skinny_gemm(a.cuda(), b_dev, (sa * sw).cuda())              # the 13-argument operator, one combined scale
+        cases.append((f"{name} m={m} row-major", out, a, sa))
+        if m == 8:
+            print(f"{name} m={m} packed: plan {plan_table.get_plan(m, n, k, True).as_dict()}", flush=True)
+            out_p = skinny_gemm_scaled(a.cuda(), pack_weight(b_dev.t()), sa.cuda(), sw_dev)
+            cases.append((f"{name} m={m} packed", out_p, a, sa))
+    torch.cuda.synchronize()
+    _check_columns_against_oracle(cases, b.t(), sw)
+
+
+def test_committed_gemm_fixtures_on_the_device():
+    """tests/golden/gemm_*.npz hold operand codes, the oracle's bf16 result and the exact integer dot products: the
+    device result, through the C ABI, must be the correctly rounded exact product up to rare one-ulp boundary cases."""
+    import glob
+    import os
+
+    import numpy as np
+    og = _oracle()
+    files = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gemm_*.npz")))
+    assert len(files) >= 3
+    for f in files:
+        z = np.load(f)
+        a = torch.from_numpy(z["a_codes"]).view(torch.float8_e4m3fn).cuda()
+        w = torch.from_numpy(z["w_codes"]).view(torch.float8_e4m3fn).cuda()
+        sa, sw = torch.from_numpy(z["scale_a"]).cuda(), torch.from_numpy(z["scale_w"]).cuda()
+        m, n = a.shape[0], w.shape[0]
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        run_ex(a, w.t(), sa, sw, out, accumulate=False)
+        got = out.cpu()
+        exact = torch.from_numpy(z["int_dots"].astype(np.float64) * 2.0 ** -18) * sa.cpu().double().reshape(-1, 1) * sw.cpu().double().reshape(1, -1)
+        err = (got.double() - exact).abs()
+        bound = og.error_bound(a.cpu(), w.cpu().t(), sa.cpu(), sw.cpu(), torch.bfloat16, exact)
+        assert (err <= bound).all(), (f, float((err / bound).max()))
+        # the exact product rounded once: the device's fp32 sums of 256..1024 cancelling terms carry an error of about
+        # 2^-17 of the result, so about one result in a hundred lands on the other side of a bf16 rounding boundary
+        differs = got.view(torch.int16) != exact.to(torch.bfloat16).view(torch.int16)
+        assert differs.float().mean() <= 0.03, (f, float(differs.float().mean()))
+        # the fixture's own result comes from the fp32 path, which scales the operands before multiplying: more boundary
+        # flips, none beyond one step
+        want = torch.from_numpy(z["out_bf16_bits"]).view(torch.bfloat16)
+        differs = got.view(torch.int16) != want.view(torch.int16)
+        assert differs.float().mean() <= 0.03, (f, float(differs.float().mean()))
+        assert ((got.double() - want.double()).abs() <= 2 * bound).all(), f   # each within `bound` of the exact product
+
+
+# ---- workspaces: one per stream, arrival counters shared by every launch on a stream -----------------------------------
+
+def _launch_ex(lib, a, b, sa, sb, out, plan, stream):
+    from hf_rocm_kernels import _capi
+    m, k = a.shape
+    st = lib.hfrk_skinny_gemm_ex(a.data_ptr(), b.data_ptr(), out.data_ptr(), sa.data_ptr(), 0 if sa.numel() == 1 else 1,
+                                 sb.data_ptr(), 0 if sb.numel() == 1 else 1, m, b.shape[1], k, b.stride(1), _capi.BF16, 0,
+                                 None if plan is None else ctypes.byref(plan), stream.cuda_stream)
+    assert st == 0, st
+
+
+def test_two_streams_run_independent_gemms():
+    """Two streams, two shapes whose row tiles are shared between workgroups (so both use workspace and counters),
+    launched interleaved without synchronisation 50 times: every result equals the one the same launch gives alone.
+    The reference's calls are independent of each other because it accumulates into the caller's output
+    (csrc/op_src/skinny_gemm/consumers/mfma_16x16x32_consumer.cu:155-163); here each stream owns a workspace."""
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    lib = _capi.load()
+    a1, b1, sa1, sw1 = generate_llama_gemm_data(8, 4096, 4096, seed=91)
+    a2, b2, sa2, sw2 = generate_llama_gemm_data(32, 4096, 14336, seed=92)
+    p1 = _capi.GemmPlan(1, 0, 1, 2, 120, 256, 16, 8 * 2 * 4096)       # wave-stream on 120 workgroups: tiles cut between them
+    p2 = _capi.GemmPlan(2, 4, 2, 1, 120, 64, 28, 8 * 4096 + 2 * 32 * 512)  # workgroup kernel, 4 x 2 waves, 120 workgroups
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    alone1 = torch.empty((8, 4096), dtype=torch.bfloat16, device="cuda")
+    alone2 = torch.empty((32, 4096), dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    _launch_ex(lib, a1, b1, sa1, sw1, alone1, p1, s1)
+    torch.cuda.synchronize()
+    _launch_ex(lib, a2, b2, sa2, sw2, alone2, p2, s2)
+    torch.cuda.synchronize()
+    check_against_oracle(alone1, a1, b1, sa1, sw1)
+    check_against_oracle(alone2, a2, b2, sa2, sw2)
+    id1, id2 = lib.hfrk_workspace_id(s1.cuda_stream), lib.hfrk_workspace_id(s2.cuda_stream)
+    assert id1 >= 0 and id2 >= 0 and id1 != id2, (id1, id2)
+    per_iter = 4
+    outs1 = [torch.full((8, 4096), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(per_iter)]
+    outs2 = [torch.full((32, 4096), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(per_iter)]
+    torch.cuda.synchronize()
+    for it in range(50):
+        for j in range(per_iter):
+            _launch_ex(lib, a1, b1, sa1, sw1, outs1[j], p1, s1)
+            _launch_ex(lib, a2, b2, sa2, sw2, outs2[j], p2, s2)
+        torch.cuda.synchronize()
+        for j in range(per_iter):
+            assert torch.equal(outs1[j], alone1), f"iteration {it}, launch {j}: stream 1 differs from its run alone"
+            assert torch.equal(outs2[j], alone2), f"iteration {it}, launch {j}: stream 2 differs from its run alone"
+            outs1[j].fill_(float("nan"))
+            outs2[j].fill_(float("nan"))
+        torch.cuda.synchronize()
+    # a stream keeps its workspace; releasing it hands the workspace to the next stream that asks
+    assert lib.hfrk_workspace_id(s1.cuda_stream) == id1
+    assert lib.hfrk_release_stream(s1.cuda_stream) == 0 and lib.hfrk_workspace_id(s1.cuda_stream) == -1
+    assert lib.hfrk_release_stream(s1.cuda_stream) == 0
+    assert lib.hfrk_reset_workspace(torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    _launch_ex(lib, a1, b1, sa1, sw1, outs1[0], p1, s1)
+    torch.cuda.synchronize()
+    assert lib.hfrk_workspace_id(s1.cuda_stream) == id1 and torch.equal(outs1[0], alone1)
+
+
+def test_back_to_back_launches_of_different_plans_share_counters_safely():
+    """Every plan of one shape uses the same arrival counters and workspace addresses with a different meaning.  300
+    launches cycling through them on one stream with no synchronisation in between: each must give the bits its plan
+    gave when it ran alone (the partial sums are exchanged past the caches and the counters reset themselves, with
+    no fence between launches)."""
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    lib = _capi.load()
+    m, n, k = 24, 1040, 4096
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=93)
+    plans = all_plans(m, n, k)
+    stream = torch.cuda.current_stream()
+    alone = []
+    for p in plans:
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        _launch_ex(lib, a, b, sa, sw, out, p, stream)
+        torch.cuda.synchronize()
+        alone.append(out)
+    check_against_oracle(alone[0], a, b, sa, sw)
+    launches = 300
+    outs = [torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in range(launches)]
+    torch.cuda.synchronize()
+    for i in range(launches):
+        _launch_ex(lib, a, b, sa, sw, outs[i], plans[(i * 7) % len(plans)], stream)
+    torch.cuda.synchronize()
+    for i in range(launches):   # stops at the first mismatch
+        j = (i * 7) % len(plans)
+        assert torch.equal(outs[i], alone[j]), f"launch {i} (plan {plans[j].as_dict()}) differs from the same plan run alone"
