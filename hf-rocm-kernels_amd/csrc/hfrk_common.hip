@@ -30,6 +30,7 @@ const char* hfrk_status_string(int status) {
         case HFRK_HIP_ERROR: return "HIP runtime error (see hfrk_last_hip_error)";
         case HFRK_NOT_INITIALISED: return "no free split-K workspace and the stream is capturing: call hfrk_init(), and launch once on further streams, first";
         case HFRK_BAD_FILE: return "plan-table file cannot be read or is not a plan table";
+        case HFRK_EXCEEDS_SCRATCH: return "the plan needs more partial sums or counters than the allocation-free entry point's scratch array holds";
         case HFRK_NO_WORKSPACE: return "too many streams hold a split-K workspace (hfrk_release_stream frees one)";
         default: return "unknown status";
     }

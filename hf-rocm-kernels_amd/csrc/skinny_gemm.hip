@@ -539,6 +539,27 @@ static int workspace_for(int dev, hipStream_t stream, Workspace* out) {
     return HFRK_SUCCESS;
 }
 
+// ---- the allocation-free entry point's scratch: one array per device, part of the code object -----------------------------
+// First kStaticWsBytes: fp32 partial sums; then kStaticCounters arrival counters.
+constexpr size_t kStaticWsBytes = (size_t)16 << 20;
+constexpr int kStaticCounters = 1 << 16;
+static __device__ __align__(256) unsigned char scratch[kStaticWsBytes + (size_t)kStaticCounters * sizeof(int)];
+static unsigned char* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, from hipGetSymbolAddress
+
+// `scratch` names the array on the host side only; kernels and HIP calls take the address looked up here.
+static int static_scratch(int dev, unsigned char** out) {
+    if (dev < 0 || dev >= kMaxDevices) return HFRK_BAD_SHAPE;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        HFRK_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) return HFRK_HIP_ERROR;
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return HFRK_SUCCESS;
+}
+
 constexpr int lds_bytes_for(int mt, int wk, int ch, int rt = 1) {
     return kGemmWaves * rt * kTileBytes + 2 * 16 * mt * (256 * wk * ch);
 }
@@ -796,10 +817,20 @@ static int choose_plan(int m, int n, int k, bool packed, hfrk_gemm_plan* plan) {
     return make_plan(m, n, k, plan);
 }
 
+// Workspace bytes and arrival counters a plan's kernel may touch (the kernels' own slot arithmetic, 1 KB per 16x16 fp32 tile).
+static size_t plan_ws_bytes(const hfrk_gemm_plan& p) {
+    if (p.wn == 0) return (size_t)p.grid * 2 * (p.wk * ((p.ch + 3) / 4)) * 1024;  // two slots per workgroup, row tiles x activation tiles
+    if (p.wn == -1) return p.slabs > 1 ? (size_t)p.panels * p.slabs * p.m_tiles * 1024 : 0;  // one share per unit and activation tile
+    return (size_t)p.grid * 2 * (p.wn * p.m_tiles) * 1024;  // two slots per workgroup, a panel's tiles x activation tiles
+}
+static long plan_counters(const hfrk_gemm_plan& p) { return p.wn == -1 ? (long)p.panels * p.m_tiles : p.panels; }
+
 // D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
+// use_static: partial sums and counters go to this device's `scratch` array instead of the stream's workspace.
 static int gemm_launch(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
                        const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k, int b_stride,
-                       int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream, bool packed = false) {
+                       int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream, bool packed = false,
+                       bool use_static = false) {
     if (packed) b_stride = k;
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
@@ -837,8 +868,27 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
     Workspace st;
-    const int rc = workspace_for(dev, stream, &st);
-    if (rc != HFRK_SUCCESS) return rc;
+    size_t ws_bytes = kWsFloats * sizeof(float);
+    long counters = kMaxPanels;
+    if (use_static) {
+        unsigned char* ptr = nullptr;
+        const int rc = static_scratch(dev, &ptr);
+        if (rc != HFRK_SUCCESS) return rc;
+        st.ws = reinterpret_cast<float*>(ptr);
+        st.counters = reinterpret_cast<int*>(ptr + kStaticWsBytes);
+        ws_bytes = kStaticWsBytes;
+        counters = kStaticCounters;
+    } else {
+        const int rc = workspace_for(dev, stream, &st);
+        if (rc != HFRK_SUCCESS) return rc;
+    }
+    if (plan_ws_bytes(p) > ws_bytes || plan_counters(p) > counters) return use_static ? HFRK_EXCEEDS_SCRATCH : HFRK_BAD_SHAPE;
+    if (use_static) {
+        // The array keeps whatever the last call (or a launch that never finished) left: the counters of this plan start at zero.
+        const int count = (int)plan_counters(p);
+        hipLaunchKernelGGL(zero_ints_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, st.counters, count);
+        HFRK_HIP_TRY(hipGetLastError());
+    }
 
     GemmArgs args;
     args.A = static_cast<const uint8_t*>(A);
@@ -863,7 +913,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.chunks_q = args.units / p.grid;
     args.chunks_r = args.units % p.grid;
     args.ws = st.ws;
-    args.ws_bytes = (uint32_t)(kWsFloats * sizeof(float));
+    args.ws_bytes = (uint32_t)ws_bytes;
     args.counters = st.counters;
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, p.lds_bytes, stream);
@@ -889,6 +939,12 @@ int hfrk_init(void) {
     while ((int)d.pool.size() < hfrk::kInitialWorkspaces) {
         const int rc = hfrk::grow_pool(d);
         if (rc != HFRK_SUCCESS) return rc;
+    }
+    if (hfrk::g_scratch_ptr[dev] == nullptr) {  // this device's copy of the allocation-free entry point's array
+        void* ptr = nullptr;
+        HFRK_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(hfrk::scratch)));
+        if (ptr == nullptr) return HFRK_HIP_ERROR;
+        hfrk::g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
     }
     return HFRK_SUCCESS;
 }
@@ -992,6 +1048,13 @@ int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scal
                         int accumulate, const hfrk_gemm_plan* plan, void* stream) {
     return hfrk::gemm_launch(A, B, D, accumulate ? D : nullptr, scale_a, sa_stride, scale_b, sb_stride, nullptr, m, n, k,
                              b_stride, d_dtype, HFRK_EPILOGUE_NONE, plan, static_cast<hipStream_t>(stream));
+}
+
+int hfrk_skinny_gemm_noalloc(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
+                             const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
+                             int accumulate, const hfrk_gemm_plan* plan, void* stream) {
+    return hfrk::gemm_launch(A, B, D, accumulate ? D : nullptr, scale_a, sa_stride, scale_b, sb_stride, nullptr, m, n, k,
+                             b_stride, d_dtype, HFRK_EPILOGUE_NONE, plan, static_cast<hipStream_t>(stream), false, true);
 }
 
 int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,

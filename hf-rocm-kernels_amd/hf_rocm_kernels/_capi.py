@@ -24,6 +24,7 @@ HIP_ERROR = 10
 NOT_INITIALISED = 11
 BAD_FILE = 12
 NO_WORKSPACE = 13
+EXCEEDS_SCRATCH = 14
 
 # enum hfrk_dtype
 F16 = 0
@@ -68,6 +69,7 @@ SIGNATURES = {
     "hfrk_plan_table_clear": (_i, []),
     "hfrk_skinny_gemm": (_i, [_p, _p, _p, _p] + [_i] * 14 + [_p]),
     "hfrk_skinny_gemm_ex": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
+    "hfrk_skinny_gemm_noalloc": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_packed_weight_bytes": (ctypes.c_size_t, [_i, _i]),
     "hfrk_pack_weight": (_i, [_p, _i, _i, _p, _i, _i, _p]),

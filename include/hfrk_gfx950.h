@@ -38,7 +38,8 @@ enum hfrk_status {
     HFRK_HIP_ERROR = 10,                    /* a HIP runtime call failed; hfrk_last_hip_error() has the code */
     HFRK_NOT_INITIALISED = 11,              /* workspace missing and the stream is capturing (call hfrk_init first) */
     HFRK_BAD_FILE = 12,                     /* a plan-table file that cannot be read or is not a plan table */
-    HFRK_NO_WORKSPACE = 13                  /* more streams hold a split-K workspace than the library allows (hfrk_release_stream) */
+    HFRK_NO_WORKSPACE = 13,                 /* more streams hold a split-K workspace than the library allows (hfrk_release_stream) */
+    HFRK_EXCEEDS_SCRATCH = 14               /* hfrk_skinny_gemm_noalloc: the plan needs more than the built-in scratch array holds */
 };
 
 /* Element types of 16-bit tensors. */
@@ -161,6 +162,24 @@ int hfrk_skinny_gemm(const void* A, const void* B, void* D, const float* scale_t
 int hfrk_skinny_gemm_ex(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
                         const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
                         int accumulate, const hfrk_gemm_plan* plan, void* stream);
+
+/* hfrk_skinny_gemm_ex for callers that cannot allocate and cannot let the library allocate on their behalf: code under
+ * HIP graph capture that has not run hfrk_init, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference.  Same arguments and bit-identical results; the partial sums and arrival counters go to an array that is
+ * part of the library's code object (16 MB + 65536 counters, 16.25 MB on every device the library runs on, held until
+ * the process ends) instead of a workspace from the pool, so the call performs no hipMalloc / hipFree and nothing that
+ * allocates.
+ * Limits: the plan (the caller's, or the library's choice for the shape) may need at most 16 MB of partial sums
+ * (1 KB per 16x16 tile a workgroup may have to hand over: 2 x grid x row tiles x activation tiles for the streaming
+ * kernels) and 65536 counters (n <= 262144).  Everything the planner and the shipped plan tables choose fits (their
+ * largest: 8 row waves x 4 activation tiles on 256 workgroups); explicit plans with 16 row tiles per panel at m > 32 or
+ * grids above 256 may not, and return HFRK_EXCEEDS_SCRATCH before anything is launched.
+ * All calls on one device share the array: calls that overlap on a device (two streams, two threads) race; order them
+ * on one stream.  Each call first clears the counters its plan uses (a small kernel on `stream`), so a launch that
+ * never finished leaves nothing behind. */
+int hfrk_skinny_gemm_noalloc(const void* A, const void* B, void* D, const float* scale_a, int sa_stride,
+                             const float* scale_b, int sb_stride, int m, int n, int k, int b_stride, int d_dtype,
+                             int accumulate, const hfrk_gemm_plan* plan, void* stream);
 
 /* The GEMM with what the decoder block does around it folded in (no reference counterpart as one call; it stands
  * for skinny_gemm followed by swiglu in hf_rocm_kernels/combined_ops/llama_mlp.py:43-56, and for the residual add
