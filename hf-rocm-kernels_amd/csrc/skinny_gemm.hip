@@ -618,6 +618,40 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     return fill_stream_plan(m, n, k, row_tiles, false, 0, plan);
 }
 
+// m <= 16: every workgroup owns a band of weight rows (4-row units dealt out evenly) and all of k (skinny_gemm_rows.hip).
+// plan: wn = -2, wk = matrix tiles per chunk, ch = activation loads, panels = 4-row units, slabs = k / 256.
+static int fill_rows_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk_gemm_plan* plan) {
+    const int act_loads = (m + 3) / 4;
+    if (m > kRowsMaxM || !rows_variant_exists(act_loads, row_tiles) || k < 512) return HFRK_INVALID_CONFIG;
+    const long units = (n + 3) / 4;
+    long grid = grid_hint > 0 ? grid_hint : kNumCU;
+    if (grid > units) grid = units;
+    if (grid >= 8 && grid_hint <= 0) grid -= grid % 8;
+    plan->m_tiles = 1;
+    plan->wn = -2;
+    plan->wk = row_tiles;
+    plan->ch = act_loads;
+    plan->grid = (int)grid;
+    plan->panels = (int)units;
+    plan->slabs = k / 256;
+    plan->lds_bytes = rows_lds_bytes(row_tiles);
+    return HFRK_SUCCESS;
+}
+
+// The planner takes the row-split decomposition when the 4-row units deal out evenly: at least one per workgroup and the
+// busiest workgroup at most a tenth above the mean (on 2304 x 16384, 2.25 units per workgroup, splitting K between
+// workgroups is the better cut).  Two matrix tiles per chunk from 9 rows on, once a band has 24 rows to fill them
+// (57344 x 8192 at 16 rows: 72.3 against 79.5 us; 4096 x 4096, 16 rows per band: 5.7 against 6.3 the other way).
+static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (m > kRowsMaxM || k < 512) return HFRK_INVALID_CONFIG;
+    const long units = (n + 3) / 4;
+    if (units < kNumCU) return HFRK_INVALID_CONFIG;
+    const long busiest = (units + kNumCU - 1) / kNumCU;
+    if (units * 10 < busiest * kNumCU * 9) return HFRK_INVALID_CONFIG;
+    const int row_tiles = (m >= 9 && 4 * busiest >= 24) ? 2 : 1;
+    return fill_rows_plan(m, n, k, row_tiles, 0, plan);
+}
+
 // 17 <= m <= 64 (valid from 1): the waves of a workgroup split K windows of 8*wave_k bytes, activations in registers
 // (skinny_gemm_ksplit.hip).  wave_k 512 keeps twice the bytes in flight and halves the window count, 256 makes
 // twice the units: take the one whose busiest workgroup streams fewer bytes.
@@ -654,8 +688,9 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 
 // Which decomposition for which shape.  The rules are measurements on MI355X over the Llama-3 8B/70B linears
 // (sweeps of every decomposition at m = 1..64), not a model:
-//   m <= 16          wave-stream kernel (activations per wave from L2: cheap up to 16 rows); K-split kernel for weights
-//                    of at most 2048 chunks (8 MB) when one window of it covers k
+//   m <= 16          row-split kernel (a band of weight rows and all of k per workgroup) when the rows deal out evenly,
+//                    else the wave-stream kernel (chunk runs that may split a tile's k between workgroups); K-split kernel
+//                    for weights of at most 2048 chunks (8 MB) when one window of it covers k
 //   m  > 16          K-split kernel (activations in registers) when one window of it covers k; otherwise the
 //                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
 //                    4 row waves x 2 K waves almost everywhere; 2 x 4 for narrow weights (n <= 2048: more K parallelism
@@ -679,7 +714,7 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
     return HFRK_SUCCESS;
 }
 
-static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = false) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
     if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     // k = 1024 is four chunks per row tile: too few for the wave-stream split and half a K-split window.  Four K waves
@@ -692,6 +727,9 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         // (2048 x 2048: 3.8 against 5.2 us; 2048 x 4096: 5.0 against 5.8).
         const long chunks = (long)((n + 15) / 16) * (k / 256);
         if (chunks <= (long)kNumCU * kGemmWaves && make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
+        // Bands of rows per workgroup: nothing crosses workgroups and the end of the launch is short (0.3-1.3 us less than
+        // the wave-stream split on every Llama-3 8B / 70B projection at 1..16 rows).
+        if (!packed && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // (row-major weights only)
         return make_stream_plan(m, n, k, plan);
     }
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
@@ -707,8 +745,18 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     return HFRK_BAD_SHAPE;
 }
 
-static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p) {
+static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p, bool packed = false) {
     if (swiglu && p->wn != 0) return HFRK_INVALID_CONFIG;  // the fused epilogue exists in the wave-stream kernel only
+    if (p->wn == -2) {  // row-split decomposition: wk = matrix tiles per chunk, ch = activation loads
+        if (packed || swiglu) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
+        if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
+        if (p->m_tiles != 1 || p->panels != (n + 3) / 4 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
+        if (p->grid < 1 || p->grid > kMaxGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
+        if (p->lds_bytes != rows_lds_bytes(p->wk)) return HFRK_INVALID_CONFIG;
+        // a band's chunk indices stay far below 2^32 / slabs (the kernel divides by multiplying with a reciprocal)
+        if (((long)p->panels / p->grid / (4 * p->wk) + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;
+        return HFRK_SUCCESS;
+    }
     if (p->wn == -1) {  // K-split decomposition: wk = wave_k / 256
         hfrk_gemm_plan want;
         const int rc = fill_ksplit_plan(m, n, k, p->wk * 256, p->grid, &want);
@@ -808,22 +856,23 @@ static int choose_plan(int m, int n, int k, bool packed, hfrk_gemm_plan* plan) {
         for (int mm = m; mm <= top && !g_plan_table.empty(); ++mm) {
             if (!plan_key(mm, n, k, packed, &key)) break;
             const auto it = g_plan_table.find(key);
-            if (it != g_plan_table.end() && check_plan(m, n, k, false, &it->second) == HFRK_SUCCESS) {
+            if (it != g_plan_table.end() && check_plan(m, n, k, false, &it->second, packed) == HFRK_SUCCESS) {
                 *plan = it->second;
                 return HFRK_SUCCESS;
             }
         }
     }
-    return make_plan(m, n, k, plan);
+    return make_plan(m, n, k, plan, packed);
 }
 
 // Workspace bytes and arrival counters a plan's kernel may touch (the kernels' own slot arithmetic, 1 KB per 16x16 fp32 tile).
 static size_t plan_ws_bytes(const hfrk_gemm_plan& p) {
+    if (p.wn == -2) return 0;  // row-split: nothing crosses workgroups
     if (p.wn == 0) return (size_t)p.grid * 2 * (p.wk * ((p.ch + 3) / 4)) * 1024;  // two slots per workgroup, row tiles x activation tiles
     if (p.wn == -1) return p.slabs > 1 ? (size_t)p.panels * p.slabs * p.m_tiles * 1024 : 0;  // one share per unit and activation tile
     return (size_t)p.grid * 2 * (p.wn * p.m_tiles) * 1024;  // two slots per workgroup, a panel's tiles x activation tiles
 }
-static long plan_counters(const hfrk_gemm_plan& p) { return p.wn == -1 ? (long)p.panels * p.m_tiles : p.panels; }
+static long plan_counters(const hfrk_gemm_plan& p) { return p.wn == -2 ? 0 : p.wn == -1 ? (long)p.panels * p.m_tiles : p.panels; }
 
 // D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
 // use_static: partial sums and counters go to this device's `scratch` array instead of the stream's workspace.
@@ -854,7 +903,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     hfrk_gemm_plan p;
     if (user_plan) {
         p = *user_plan;
-        const int rc = check_plan(m, swiglu ? n / 2 : n, k, swiglu, &p);
+        const int rc = check_plan(m, swiglu ? n / 2 : n, k, swiglu, &p, packed);
         if (rc != HFRK_SUCCESS) return rc;
     } else {
         const int rc = swiglu ? fill_stream_plan(m, n / 2, k, 1, false, 0, &p) : choose_plan(m, n, k, packed, &p);
@@ -870,7 +919,11 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     Workspace st;
     size_t ws_bytes = kWsFloats * sizeof(float);
     long counters = kMaxPanels;
-    if (use_static) {
+    if (plan_ws_bytes(p) == 0 && plan_counters(p) == 0) {
+        ws_bytes = 0;  // nothing crosses workgroups under this plan: no workspace is taken
+        counters = 0;
+        use_static = false;
+    } else if (use_static) {
         unsigned char* ptr = nullptr;
         const int rc = static_scratch(dev, &ptr);
         if (rc != HFRK_SUCCESS) return rc;
@@ -915,6 +968,20 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.ws = st.ws;
     args.ws_bytes = (uint32_t)ws_bytes;
     args.counters = st.counters;
+    if (p.wn == -2) {
+        const int per_tile = 4 * p.wk;  // units a tile can hold
+        args.rows_q = p.panels / p.grid;
+        args.rows_r = p.panels % p.grid;
+        auto geometry = [&](int units, int* tiles, int* base, int* extra) {
+            *tiles = (units + per_tile - 1) / per_tile;
+            *base = *tiles ? units / *tiles : 0;
+            *extra = *tiles ? units % *tiles : 0;
+        };
+        geometry(args.rows_q + 1, &args.tiles_a, &args.base_a, &args.extra_a);
+        geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
+        args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)p.slabs - 1) / (uint64_t)p.slabs);
+        return launch_rows_kernel(args, p.ch, p.wk, p.lds_bytes, stream);
+    }
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, p.lds_bytes, stream);
     switch (p.m_tiles) {
@@ -1012,7 +1079,7 @@ int hfrk_plan_table_set(int m, int n, int k, int packed, const hfrk_gemm_plan* p
     uint64_t key;
     if (!hfrk::plan_key(m, n, k, packed, &key)) return HFRK_BAD_SHAPE;
     if (plan) {
-        const int rc = hfrk::check_plan(m, n, k, false, plan);
+        const int rc = hfrk::check_plan(m, n, k, false, plan, packed != 0);
         if (rc != HFRK_SUCCESS) return rc;
     }
     std::lock_guard<std::mutex> lock(hfrk::g_plan_mutex);

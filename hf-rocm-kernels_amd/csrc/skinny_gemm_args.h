@@ -28,6 +28,11 @@ struct GemmArgs {
     int d_dtype;             // dtype of D; with the SwiGLU epilogue the 16-bit dtype the projections are rounded to
     int panels, slabs, units, grid;  // units = panels * slabs
     int chunks_q, chunks_r;  // stream kernel: (panels * slabs) / grid and % grid
+    // row-split kernel: 4-row units per workgroup (rows_q, the first rows_r workgroups one more), and for both band
+    // heights (a: rows_q + 1 units, b: rows_q) the tiles of a band, units per tile and how many tiles have one more
+    int rows_q, rows_r;
+    int tiles_a, base_a, extra_a, tiles_b, base_b, extra_b;
+    uint32_t kc_magic;       // ceil(2^32 / slabs): i / slabs == umulhi(i, kc_magic) for the chunk indices of a band
     float* ws;               // fp32 partial sums that cross workgroups
     uint32_t ws_bytes;       // size of ws: accesses beyond it are dropped by the buffer range check
     int* counters;           // arrival counters, zero between launches
@@ -46,6 +51,15 @@ constexpr int stream_lds_bytes(int act_loads, int row_tiles) {
 constexpr bool stream_variant_exists(int act_loads, int row_tiles, bool swiglu = false) {
     return swiglu ? (row_tiles == 2 && act_loads >= 1 && act_loads <= 4)
                   : (row_tiles == 1 && act_loads >= 1 && act_loads <= 4) || (row_tiles == 2 && act_loads >= 3 && act_loads <= 8);
+}
+
+// row-split wave-stream kernel (m <= 16), skinny_gemm_rows.hip: every workgroup owns a band of weight rows and all of k;
+// act_loads = ceil(m/4), row_tiles = 16-row matrix tiles per chunk (1 or 2).  Needs k >= 512.
+int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream);
+constexpr int kRowsMaxM = 16;
+constexpr int rows_lds_bytes(int row_tiles) { return kGemmWaves * (row_tiles + 1) * kTileBytes; }
+constexpr bool rows_variant_exists(int act_loads, int row_tiles) {
+    return act_loads >= 1 && act_loads <= 4 && (row_tiles == 1 || row_tiles == 2);
 }
 
 // K-split kernel (skinny_gemm_ksplit.hip): the 8 waves of a workgroup split a K window of 8*wave_k bytes

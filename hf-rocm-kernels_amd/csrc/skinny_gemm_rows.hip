@@ -1,0 +1,332 @@
+// FP8 skinny GEMM, m <= 16, weights of at least a few rows per workgroup: the row-split wave-stream kernel.
+//
+// Every workgroup owns a contiguous band of weight rows and all of K for them, so no sum ever crosses workgroups: there
+// is no workspace, no arrival counter and no memory round trip after the weight stream ends.  The weight rows are dealt
+// out in units of 4 rows (what one 16-byte load instruction of a wave covers: 4 rows x 256 bytes), `rows_q` units per
+// workgroup and one more for the first `rows_r`; a band is cut into tiles of at most 4*RT units of nearly equal height
+// (RT = 1 or 2 matrix-core tiles of 16 rows), e.g. 40 rows = 16 + 12 + 12.  Loads of a short tile's missing units are
+// out of the buffer's range and cost no traffic.  Inside the workgroup the sequence of chunks (tile-major, K fastest;
+// a chunk is one tile x 256 K-bytes) is split evenly over the 8 waves, each wave streams its run exactly like the
+// wave-stream kernel of skinny_gemm_stream.hip (private swizzled LDS tiles, v_mfma_f32_16x16x128_f8f6f4, the next
+// chunk requested as soon as the registers are free).
+//
+// A launch of this kind lives 5-70 us and a lone wave retires one instruction every 2-4 ns, so what is not streaming is
+// instruction count on the critical path.  Two places matter and are kept short:
+//  * before the first request: the partition is a handful of scalar multiplies (the tile geometry of both band heights
+//    and the reciprocal of the chunk count come from the host), and everything the end of the kernel will need -- which
+//    wave finishes which tile, whose partial sums it adds, where the results go, the old D values and channel scales --
+//    is worked out after the first request, while it is in flight;
+//  * after the last matrix instruction: a wave whose run starts inside a tile leaves its partial 16x16 tile in LDS, one
+//    barrier, and the wave whose run holds the tile's first chunk adds the partials of the waves after it (a
+//    precomputed bit mask says which), scales, rounds once and stores.  Each wave finishes at most one tile there.
+// Sums are added in wave order: results are bit-reproducible.
+//
+// Replaces, for these shapes, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and
+// consumers (producers/n_full_tiles.cu:4-127, consumers/mfma_16x16x32_consumer.cu:1-168,
+// consumers/smfma_16x16x64_consumer.cu:1-158).
+#include "skinny_gemm_args.h"
+
+namespace hfrk {
+
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+// two fp32 -> two 16-bit values in one register, round to nearest even (v_cvt_pk_bf16_f32 / v_cvt_f16_f32)
+__device__ __forceinline__ uint32_t pack16(float lo, float hi, bool bf16) {
+    const v2f v = {lo, hi};
+    return bf16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2bf))
+                : __builtin_bit_cast(uint32_t, __builtin_convertvector(v, v2h));
+}
+
+// MA = ceil(m/4): 16-byte activation loads per lane and chunk (rows 4t .. 4t+3), RT = 16-row matrix tiles per chunk.
+template <int MA, int RT>
+__global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const GemmArgs a) {
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    constexpr int kWaveLds = (RT + 1) * kTileBytes;  // RT weight tiles, one activation tile
+    constexpr int kSlotStride = kWaveLds / 16;       // in v4f
+
+    extern __shared__ __align__(16) uint8_t lds[];
+    // A wave's partial sums (RT x 64 lanes x 16 bytes) go to the start of its own weight tiles, which are dead by then.
+    v4f* const slots = reinterpret_cast<v4f*>(lds);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+
+    // ---- this workgroup's band of rows and this wave's run of chunks -----------------------------------------------
+    const int G = a.grid;
+    const int b = blockIdx.x;
+    const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;  // XCD x owns logical ids [x*G/8, (x+1)*G/8)
+    const bool tall = g < a.rows_r;                                    // one unit more than the others
+    const int u0 = g * a.rows_q + min(g, a.rows_r);                    // first 4-row unit of the band
+    const int T = tall ? a.tiles_a : a.tiles_b;                        // tiles of the band
+    const int ubase = tall ? a.base_a : a.base_b;                      // units per tile, the first `uextra` tiles one more
+    const int uextra = tall ? a.extra_a : a.extra_b;
+    const int KC = a.slabs;                                            // 256-byte chunks per tile
+    const int TC = T * KC;
+    const int i0 = (wv * TC) >> 3, i1 = ((wv + 1) * TC) >> 3;          // chunks [i0, i1) of the band, tile-major
+    const int count = i1 - i0;
+    int tile = (int)__umulhi((uint32_t)i0, a.kc_magic);               // i0 / KC
+    int kc = i0 - tile * KC;
+
+    // ---- first request, as early as possible ---------------------------------------------------------------------
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
+    const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
+    const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
+    v4i wq[4 * RT], aq[MA];
+    int itile = tile, ikc = kc;                                        // chunk being requested
+    int iunits = ubase + (itile < uextra ? 1 : 0);                     // its tile's height in units
+    int irow0 = 4 * (u0 + itile * ubase + min(itile, uextra));        // its tile's first row
+    uint32_t irow_off = (uint32_t)irow0 * (uint32_t)a.b_stride;
+    auto issue_chunk = [&]() __attribute__((always_inline)) {
+        const uint32_t kbyte = (uint32_t)ikc * 256u;
+#pragma unroll
+        for (int t = 0; t < MA; ++t)
+            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+#pragma unroll
+        for (int t = 0; t < 4 * RT; ++t) {  // unit t of the tile; a unit the tile does not have reads as zero, without traffic
+            const uint32_t off = t < iunits ? irow_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.b_stride : kOutOfRange;
+            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + off), 0, 2 /* nt */);
+        }
+    };
+    auto next_chunk = [&]() __attribute__((always_inline)) {
+        if (++ikc == KC) {
+            ikc = 0;
+            irow0 += 4 * iunits;
+            irow_off = (uint32_t)irow0 * (uint32_t)a.b_stride;
+            ++itile;
+            iunits = ubase + (itile < uextra ? 1 : 0);
+        }
+    };
+    if (count > 0) issue_chunk();
+    __builtin_amdgcn_sched_barrier(0);  // keep the set-up below behind the first request
+
+    // ---- the rest of the set-up, while the first chunk is on its way -------------------------------------------------
+    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
+    const __amdgpu_buffer_rsrc_t base_rsrc = make_rsrc(a.base, a.base ? (uint32_t)a.m * (uint32_t)a.n * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
+    const bool accumulate = a.base != nullptr;
+    const bool vec = (a.n & 3) == 0;  // then a lane's four outputs are all inside n and 8-byte aligned
+    const bool per_channel = a.scale_b && a.sb_stride;
+    const bool bf16 = a.d_dtype == HFRK_BF16;
+    // lane li holds the accumulator column of activation row li
+    const float sa = a.scale_a[(long)min(li, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+
+    uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its activation tile
+    uint8_t* const ta = tw + RT * kTileBytes;
+    int wr_off[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int row = 4 * t + lg;
+        wr_off[t] = row * 256 + ((li ^ row) << 4);
+    }
+    int rd_off[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) rd_off[h] = li * 256 + ((((8 * h + 2 * lg) ^ li) & 15) << 4);
+
+    // Old D values (accumulate mode) and per-channel scales of a tile whose first row is `row0` (aligned n only; ragged
+    // n fetches in the epilogue).  Nothing is requested when nothing is wanted.
+    struct Pre { v2i d[RT]; v4i sb[RT]; };
+    const bool want_pre = vec && (accumulate || per_channel);
+    auto prefetch = [&](int row0, int units, bool wanted) __attribute__((always_inline)) {
+        Pre p;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            p.sb[rt] = v4i{0, 0, 0, 0};
+            p.d[rt] = v2i{0, 0};
+        }
+        if (wanted && want_pre) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const int ul = 4 * rt + lg;  // this lane's unit of the tile
+                const int n0 = row0 + 4 * ul;
+                const bool ok = ul < units && n0 < a.n;
+                p.sb[rt] = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (per_channel && ok) ? n0 * 4 : (int)kOutOfRange, 0, 0);
+                p.d[rt] = __builtin_amdgcn_raw_buffer_load_b64(base_rsrc, (accumulate && ok && li < a.m) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
+            }
+        }
+        return p;
+    };
+
+    // scale, add D (accumulate mode), round once, store: lane holds D[li][n0 + v], v = 0..3, n0 = row0 + 16*rt + 4*lg
+    auto epilogue = [&](int row0, int units, const v4f (&acc)[RT], const Pre& pre) __attribute__((always_inline)) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const int ul = 4 * rt + lg;
+            const int n0 = row0 + 4 * ul;
+            const bool live = li < a.m && ul < units && n0 < a.n;
+            const uint32_t d_off = ((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u;
+            if (vec) {
+                const v4f sb = __builtin_bit_cast(v4f, pre.sb[rt]);
+                const uint32_t d0 = (uint32_t)pre.d[rt][0], d1 = (uint32_t)pre.d[rt][1];
+                float r[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) r[v] = acc[rt][v] * (per_channel ? sa * sb[v] : sa);
+                if (accumulate) {
+                    if (bf16) {
+                        r[0] += __uint_as_float(d0 << 16); r[1] += __uint_as_float(d0 & 0xffff0000u);
+                        r[2] += __uint_as_float(d1 << 16); r[3] += __uint_as_float(d1 & 0xffff0000u);
+                    } else {
+                        r[0] += f16_bits_to_float((uint16_t)d0); r[1] += f16_bits_to_float((uint16_t)(d0 >> 16));
+                        r[2] += f16_bits_to_float((uint16_t)d1); r[3] += f16_bits_to_float((uint16_t)(d1 >> 16));
+                    }
+                }
+                const v2i packed = {(int)pack16(r[0], r[1], bf16), (int)pack16(r[2], r[3], bf16)};
+                __builtin_amdgcn_raw_buffer_store_b64(packed, d_rsrc, live ? (int)d_off : (int)kOutOfRange, 0, 0);
+            } else {
+                // ragged n: 2-byte accesses whose out-of-range offsets mask the columns beyond n
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const uint32_t off = (live && n0 + v < a.n) ? d_off + 2u * v : kOutOfRange;
+                    const uint32_t old = accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(base_rsrc, (int)off, 0, 0) : 0u;
+                    const float sbv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, (live && per_channel && n0 + v < a.n) ? (n0 + v) * 4 : (int)kOutOfRange, 0, 0));
+                    float r = acc[rt][v] * (per_channel ? sa * sbv : sa);
+                    if (accumulate) r += bf16 ? bf16_bits_to_float((uint16_t)old) : f16_bits_to_float((uint16_t)old);
+                    __builtin_amdgcn_raw_buffer_store_b16((short)(pack16(r, 0.f, bf16) & 0xffffu), d_rsrc, (int)off, 0, 0);
+                }
+            }
+        }
+    };
+
+    // ---- what the end of the kernel will do, decided now ----------------------------------------------------------------
+    // A run that starts inside a tile (kb0 != 0) hands the partial sum of that tile over; a wave without chunks hands over
+    // zeros, so that the finishing wave can add by position alone.  The wave whose run holds a tile's first chunk finishes
+    // it: in the loop when the tile also ends inside the run, after the barrier when it ends in a later wave's run.
+    const int tile_h = tile, kb0 = kc;
+    const bool hand_over = count == 0 || kb0 != 0;
+    const int jl = (int)__umulhi((uint32_t)i1, a.kc_magic);  // the tile the run ends in
+    const int ke = i1 - jl * KC;                             // its chunks before the end of the run
+    const bool finisher = count > 0 && ke != 0 && jl * KC >= i0;
+    const int units_l = ubase + (jl < uextra ? 1 : 0);
+    const int row0_l = 4 * (u0 + jl * ubase + min(jl, uextra));
+    uint32_t addmask = 0;  // bit j: wave j's run starts before that tile ends, its partial belongs to it
+    {
+        const int e = (jl + 1) * KC;
+#pragma unroll
+        for (int j = 1; j < kGemmWaves; ++j)
+            if (j > wv && ((j * TC) >> 3) < e) addmask |= 1u << j;
+    }
+    const Pre pre_l = prefetch(row0_l, units_l, finisher);
+
+    // ---- streaming loop ---------------------------------------------------------------------------------------------
+    int units = iunits;                                      // geometry of the tile being multiplied
+    int row0 = 4 * (u0 + tile * ubase + min(tile, uextra));
+    Pre pre_next = prefetch(row0, units, count > 0 && kc == KC - 1 && !(kb0 != 0)), pre_cur;
+    v4f acc[RT], part_h[RT];
+#pragma unroll
+    for (int u = 0; u < RT; ++u) acc[u] = part_h[u] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < count; ++i) {
+#pragma unroll
+        for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
+#pragma unroll
+        for (int t = 0; t < 4 * RT; ++t) *reinterpret_cast<v4i*>(tw + (t / 4) * kTileBytes + wr_off[t % 4]) = wq[t];
+        pre_cur = pre_next;
+        if (i + 1 < count) {  // registers are free again: request the next chunk before the LDS reads and MFMAs
+            next_chunk();
+            issue_chunk();
+            // the chunk that ends a tile this wave finishes in the loop brings the tile's D along
+            pre_next = prefetch(irow0, iunits, ikc == KC - 1 && !(itile == tile_h && kb0 != 0));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // every operand of the chunk is requested from LDS before the first MFMA
+        v8i wop[2][RT], aop[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const v4i lo = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + rd_off[h]);
+                const v4i hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
+                wop[h][rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+            const v4i lo = *reinterpret_cast<const v4i*>(ta + rd_off[h]);
+            const v4i hi = *reinterpret_cast<const v4i*>(ta + (rd_off[h] ^ 16));
+            aop[h] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests above ahead of the MFMAs below
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                acc[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h][rt], aop[h], acc[rt], 0, 0, 0, 0, 0, 0);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (++kc == KC) {  // a tile ends inside this wave's run
+            if (tile == tile_h && kb0 != 0) {  // its first chunks belong to an earlier wave
+#pragma unroll
+                for (int u = 0; u < RT; ++u) part_h[u] = acc[u];
+            } else {
+                epilogue(row0, units, acc, pre_cur);  // all of it was ours
+            }
+#pragma unroll
+            for (int u = 0; u < RT; ++u) acc[u] = v4f{0.f, 0.f, 0.f, 0.f};
+            kc = 0;
+            row0 += 4 * units;
+            ++tile;
+            units = ubase + (tile < uextra ? 1 : 0);
+        }
+    }
+    // a run that lies inside one tile that began in an earlier wave: everything it has is that tile's partial sum
+    if (count > 0 && kc != 0 && tile == tile_h && kb0 != 0) {
+#pragma unroll
+        for (int u = 0; u < RT; ++u) part_h[u] = acc[u];
+    }
+
+    // ---- combine the partial tiles of this workgroup ----------------------------------------------------------------
+    // Every wave leaves a partial sum (zeros when it has none to hand over), so that the finishing wave can read all seven
+    // slots at once and add each with a factor of one or zero: no select, no branch, exact.
+#pragma unroll
+    for (int u = 0; u < RT; ++u) slots[wv * kSlotStride + u * 64 + lane] = hand_over ? part_h[u] : v4f{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    if (!finisher) return;
+    v4f other[kGemmWaves][RT];
+#pragma unroll
+    for (int j = 1; j < kGemmWaves; ++j)
+#pragma unroll
+        for (int u = 0; u < RT; ++u) other[j][u] = slots[j * kSlotStride + u * 64 + lane];
+#pragma unroll
+    for (int j = 1; j < kGemmWaves; ++j) {
+        const float f = (addmask >> j) & 1u ? 1.0f : 0.0f;
+#pragma unroll
+        for (int u = 0; u < RT; ++u)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[u][v] = __builtin_fmaf(other[j][u][v], f, acc[u][v]);
+    }
+    epilogue(row0_l, units_l, acc, pre_l);
+}
+
+template <int MA, int RT>
+static int launch_rows_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
+    auto kern = skinny_gemm_rows_kernel<MA, RT>;
+    static bool attr_done[kMaxDevices] = {};
+    int dev = 0;
+    HFRK_HIP_TRY(hipGetDevice(&dev));
+    if (dev >= 0 && dev < kMaxDevices && !attr_done[dev]) {
+        HFRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        attr_done[dev] = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(args.grid), dim3(kGemmThreads), lds_bytes, stream, args);
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}
+
+int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream) {
+    if (!rows_variant_exists(act_loads, row_tiles) || lds_bytes != rows_lds_bytes(row_tiles)) return HFRK_INVALID_CONFIG;
+#define HFRK_ROWS_CASE(MA_)                                                                \
+    case MA_:                                                                              \
+        return row_tiles == 1 ? launch_rows_one<MA_, 1>(args, lds_bytes, stream)           \
+                              : launch_rows_one<MA_, 2>(args, lds_bytes, stream);
+    switch (act_loads) {
+        HFRK_ROWS_CASE(1)
+        HFRK_ROWS_CASE(2)
+        HFRK_ROWS_CASE(3)
+        HFRK_ROWS_CASE(4)
+    }
+#undef HFRK_ROWS_CASE
+    return HFRK_INVALID_CONFIG;
+}
+
+}  // namespace hfrk

@@ -65,6 +65,11 @@ def all_plans(m, n, k):
             groups = (n + 16 * rt - 1) // (16 * rt)
             for grid in sorted({min(g, groups * kc) for g in (256, 200, 7, 512, 1)}):
                 plans.append(_capi.GemmPlan((ma + 3) // 4, 0, rt, ma, grid, groups, kc, 8 * (rt + (ma + 3) // 4) * 4096))
+    if m <= 16 and k >= 512:  # row-split decomposition: bands of rows per workgroup, cut into tiles of different heights
+        units = (n + 3) // 4
+        for rt in (1, 2):
+            for grid in sorted({min(g, units) for g in (256, 200, 7, 512, 1, 77)}):
+                plans.append(_capi.GemmPlan(1, -2, rt, (m + 3) // 4, grid, units, k // 256, 8 * (rt + 1) * 4096))
     for wave_k in (256, 512, 1024):  # K-split decomposition
         if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
             tiles, windows = (n + 15) // 16, k // (8 * wave_k)

@@ -112,10 +112,80 @@ def _emulate(plan, n, k):
     return cover, contributors, ub
 
 
+def _emulate_rows(plan):
+    """Replays the row-split kernel's arithmetic on the host: bands of 4-row units per workgroup, tiles of nearly equal
+    height per band, chunk runs per wave, and the end-of-kernel roles (who hands a partial over, who finishes which tile,
+    whose partials it adds).  Returns nothing; asserts that every (unit, K chunk) is multiplied exactly once and every
+    tile is finished exactly once from exactly the partials that exist."""
+    G, units, KC, per_tile = plan.grid, plan.panels, plan.slabs, 4 * plan.wk
+    q, r = divmod(units, G)
+    magic = ((1 << 32) + KC - 1) // KC
+    assert magic < (1 << 32)
+    cover = [[0] * KC for _ in range(units)]
+    for g in range(G):
+        nu, u0 = q + (1 if g < r else 0), g * q + min(g, r)
+        assert nu >= 1, "empty workgroup"
+        T = -(-nu // per_tile)
+        base, extra = nu // T, nu % T
+        TC = T * KC
+        runs = [((w * TC) >> 3, ((w + 1) * TC) >> 3) for w in range(8)]
+        assert runs[0][0] == 0 and runs[-1][1] == TC and all(a[1] == b[0] for a, b in zip(runs, runs[1:]))
+        pieces = [[] for _ in range(T)]  # waves that multiply chunks of tile j, in order
+        for w, (i0, i1) in enumerate(runs):
+            for i in (i0, i1):
+                assert (i * magic) >> 32 == i // KC  # the kernel divides by multiplying with the reciprocal
+            for i in range(i0, i1):
+                j, kc = divmod(i, KC)
+                first, height = j * base + min(j, extra), base + (1 if j < extra else 0)
+                assert 1 <= height <= per_tile
+                for t in range(height):
+                    cover[u0 + first + t][kc] += 1
+                if not pieces[j] or pieces[j][-1] != w:
+                    pieces[j].append(w)
+        assert sum(base + (1 if j < extra else 0) for j in range(T)) == nu
+        finished = [0] * T
+        for w, (i0, i1) in enumerate(runs):
+            count, kb0 = i1 - i0, i0 % KC
+            for j in range(T):  # tiles that begin and end inside the run: finished in the loop, by this wave alone
+                if count > 0 and j * KC >= i0 and (j + 1) * KC <= i1:
+                    finished[j] += 1
+                    assert pieces[j] == [w]
+            jl = i1 // KC
+            ke = i1 - jl * KC
+            if count > 0 and ke != 0 and jl * KC >= i0:  # finishes tile jl after the barrier
+                finished[jl] += 1
+                added = [x for x in range(1, 8) if x > w and ((x * TC) >> 3) < (jl + 1) * KC]
+                for x in added:  # each hands over: an empty run (zeros), or a run that starts inside tile jl
+                    x0, x1 = runs[x]
+                    assert x1 == x0 or (x0 % KC != 0 and x0 // KC == jl), (g, w, x)
+                assert [x for x in added if runs[x][1] > runs[x][0]] == [x for x in pieces[jl] if x != w], (g, w, jl)
+            if count > 0 and kb0 != 0:  # hands the partial of its first tile over: somebody before it must finish that tile
+                assert pieces[i0 // KC][0] < w
+        assert finished == [1] * T, (g, finished)
+    assert all(c == 1 for row in cover for c in row)
+
+
+@pytest.mark.parametrize("rt", [1, 2])
+@pytest.mark.parametrize("n,k,grid", [(4096, 4096, 256), (6144, 4096, 256), (10240, 8192, 256), (10240, 8192, 512), (57344, 8192, 256),
+                                      (4096, 14336, 256), (1000, 512, 77), (1000, 512, 250), (50, 512, 13), (130, 1024, 7),
+                                      (2304, 16384, 256), (1024, 512, 256), (28672, 4096, 1), (8192, 28672, 1024), (8200, 768, 200)])
+def test_row_split_decomposition_on_the_host(n, k, grid, rt):
+    units = -(-n // 4)
+    plan = _capi.GemmPlan(1, -2, rt, 2, min(grid, units), units, k // 256, 8 * (rt + 1) * 4096)
+    assert _capi.load().hfrk_plan_table_set(8, n, k, 0, ctypes.byref(plan)) == _capi.SUCCESS   # the library accepts it
+    assert _capi.load().hfrk_plan_table_set(8, n, k, 0, None) == _capi.SUCCESS
+    _emulate_rows(plan)
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 33, 64])
 @pytest.mark.parametrize("n,k", SHAPES)
 def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
     plan = _capi.plan(m, n, k)
+    if plan.wn == -2:  # m <= 16, rows that deal out evenly: row-split decomposition
+        assert m <= 16 and plan.ch == (m + 3) // 4 and plan.m_tiles == 1 and plan.slabs == k // 256 and plan.panels == -(-n // 4)
+        assert plan.wk in (1, 2) and plan.lds_bytes == 8 * (plan.wk + 1) * 4096 and 1 <= plan.grid <= min(256, plan.panels)
+        _emulate_rows(plan)
+        return
     if plan.wn == 0:  # m <= 16: wave-stream decomposition
         assert m <= 16 and plan.ch == (m + 3) // 4 and plan.m_tiles == (plan.ch + 3) // 4 and plan.slabs == k // 256
         assert plan.wk in (1, 2) and (plan.wk == 2 or m <= 16) and plan.panels == -(-n // (16 * plan.wk))
@@ -317,18 +387,18 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
     m, n, k = 8, 6144, 4096
     planner = _capi.plan(m, n, k)
     assert plan_table.get_plan(m, n, k).as_dict() == planner.as_dict()
-    tuned = _capi.GemmPlan(1, 0, 1, 2, 128, planner.panels, planner.slabs, planner.lds_bytes)  # same kernel, grid 128
+    tuned = _capi.GemmPlan(1, 0, 1, 2, 128, n // 16, k // 256, 8 * 2 * 4096)  # the wave-stream kernel on 128 workgroups
     assert tuned.as_dict() != planner.as_dict()
     plan_table.set_plan(m, n, k, tuned)
     assert plan_table.get_plan(m, n, k).as_dict() == tuned.as_dict()
     assert _capi.plan(m, n, k).as_dict() == planner.as_dict()          # hfrk_skinny_gemm_plan stays the planner's rule
-    assert plan_table.get_plan(m, n, k, packed=True).as_dict() == planner.as_dict()   # another key
+    assert plan_table.get_plan(m, n, k, packed=True).as_dict() != tuned.as_dict()     # another key: the planner's choice for packed weights
     # the entry also serves the smaller m with the same activation loads (5..8), and no other
     for mm in (5, 6, 7):
         assert plan_table.get_plan(mm, n, k).as_dict() == tuned.as_dict(), mm
     for mm in (4, 9):
         assert plan_table.get_plan(mm, n, k).as_dict() == _capi.plan(mm, n, k).as_dict(), mm
-    nearer = _capi.GemmPlan(1, 0, 1, 2, 64, planner.panels, planner.slabs, planner.lds_bytes)
+    nearer = _capi.GemmPlan(1, 0, 1, 2, 64, n // 16, k // 256, 8 * 2 * 4096)
     plan_table.set_plan(6, n, k, nearer)
     assert plan_table.get_plan(5, n, k).as_dict() == nearer.as_dict()      # the nearest entry at or above m
     assert plan_table.get_plan(7, n, k).as_dict() == tuned.as_dict()
@@ -342,7 +412,7 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
     assert plan_table.get_plan(33, n, k).as_dict() == _capi.plan(33, n, k).as_dict()
     plan_table.remove_plan(32, n, k)
     # a plan that does not fit the shape is refused and changes nothing
-    bad = _capi.GemmPlan(1, 0, 1, 1, 128, planner.panels, planner.slabs, planner.lds_bytes)  # 4 rows of activations for m = 8
+    bad = _capi.GemmPlan(1, 0, 1, 1, 128, n // 16, k // 256, 8 * 2 * 4096)  # 4 rows of activations for m = 8
     with pytest.raises(RuntimeError):
         plan_table.set_plan(m, n, k, bad)
     assert _capi.load().hfrk_plan_table_set(m, n, 100, 0, ctypes.byref(tuned)) == _capi.BAD_SHAPE
@@ -437,7 +507,8 @@ def test_c_loader_installs_the_shipped_table_like_the_python_loader():
 def test_c_loader_rejects_what_is_not_a_plan_table(tmp_path):
     import json
     from hf_rocm_kernels import plan_table
-    good = {"m": 8, "n": 6144, "k": 4096, "packed": False, "plan": _capi.plan(8, 6144, 4096).as_dict(), "us": 7.25, "note": "caf\u00e9 \"x\""}
+    good = {"m": 8, "n": 6144, "k": 4096, "packed": False, "plan": _capi.GemmPlan(1, 0, 1, 2, 192, 384, 16, 65536).as_dict(),   # valid for both weight layouts
+            "us": 7.25, "note": "caf\u00e9 \"x\""}
     wrong_shape = dict(good, n=100, plan=dict(good["plan"]))        # the plan does not fit n = 100
     no_grid = dict(good, m=4, plan={k: v for k, v in good["plan"].items() if k != "grid"})
     fractional = dict(good, m=2, plan=dict(good["plan"], grid=12.5))

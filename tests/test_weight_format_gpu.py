@@ -2,6 +2,7 @@
 oracle (bit-exact: this is byte shuffling and a 256-entry code map), and the GEMM on a packed weight against the GEMM
 on the row-major weight (bit-exact: same operands, same order of sums) and against the exact product.
 Through the C ABI and through the Python surface (PackedWeight in place of `b`)."""
+import contextlib
 import ctypes
 
 import numpy as np
@@ -151,7 +152,11 @@ def test_every_plan_on_a_packed_weight_equals_the_row_major_result_bit_for_bit(m
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k, per_token=True, per_channel=True)
     packed = _pack(b.t().view(torch.uint8))
     base = torch.randn((m, n), device="cuda").to(torch.bfloat16)
-    plans = [None] + all_plans(m, n, k)
+    # the same plan gives the same bits on both layouts; left to itself the library may plan the two layouts differently
+    # (the row-split decomposition exists for row-major weights only), so the library's own choice for the packed weight
+    # is passed to both
+    from hf_rocm_kernels import plan_table
+    plans = [plan_table.get_plan(m, n, k, packed=True)] + [p for p in all_plans(m, n, k) if p.wn != -2]
     for p in plans:
         want = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         got = want.clone()
@@ -168,8 +173,10 @@ def test_float16_output_and_accumulation_on_a_packed_weight(m, n, k):
     packed = _pack(b.t().view(torch.uint8))
     base = torch.randn((m, n), device="cuda").to(torch.float16)
     want, got = base.clone(), base.clone()
-    _run_fused(a, b, want, want, sa, sw, None, 0, None, None)    # base = D itself: accumulate in place
-    _run_fused(a, b, got, got, sa, sw, None, 0, None, packed)
+    from hf_rocm_kernels import plan_table
+    plan = plan_table.get_plan(m, n, k, packed=True)             # one decomposition for both layouts
+    _run_fused(a, b, want, want, sa, sw, None, 0, plan, None)    # base = D itself: accumulate in place
+    _run_fused(a, b, got, got, sa, sw, None, 0, plan, packed)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     check_against_oracle(got, a, b, sa, sw, base=base)
 
@@ -209,6 +216,22 @@ def test_python_surface_takes_a_packed_weight_everywhere():
                            skinny_gemm_swiglu(a, b, scale, None, out_scale).view(torch.uint8))
 
 
+@contextlib.contextmanager
+def one_plan_for_both_layouts(*shapes):
+    """The same plan gives the same bits on a row-major and on a packed weight, but the library may plan the two layouts
+    differently (the row-split decomposition exists for row-major weights only).  Inside this context the row-major key of
+    each (m, n, k) holds the plan the library uses for the packed weight, so that the operators, which take no plan, can be
+    compared bit for bit."""
+    from hf_rocm_kernels import plan_table
+    try:
+        for m, n, k in shapes:
+            plan_table.set_plan(m, n, k, plan_table.get_plan(m, n, k, packed=True))
+        yield
+    finally:
+        plan_table.clear()
+        plan_table.load_from_environment()
+
+
 @pytest.mark.parametrize("fused", [False, True])
 def test_llama_mlp_block_on_packed_weights(fused):
     from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
@@ -226,8 +249,9 @@ def test_llama_mlp_block_on_packed_weights(fused):
     s_in, s_mid = torch.full((1,), 0.02, device="cuda"), torch.full((1,), 0.01, device="cuda")
     args = dict(rms_weight=wn, rms_epsilon=1e-5, gate_up_input_scale=s_in, gate_up_output_scale=(s_in * sgu).view(1),
                 down_input_scale=s_mid, down_output_scale=(s_mid * sd).view(1), add_residual=True, fused=fused)
-    want, want_res = llama_mlp_combined_ops(x, res.clone(), gate_up_weight=qgu.t(), down_weight=qd.t(), **args)
-    got, got_res = llama_mlp_combined_ops(x, res.clone(), gate_up_weight=pack_weight(qgu), down_weight=pack_weight(qd), **args)
+    with one_plan_for_both_layouts((m, 2 * inter, hidden), (m, hidden, inter)):
+        want, want_res = llama_mlp_combined_ops(x, res.clone(), gate_up_weight=qgu.t(), down_weight=qd.t(), **args)
+        got, got_res = llama_mlp_combined_ops(x, res.clone(), gate_up_weight=pack_weight(qgu), down_weight=pack_weight(qd), **args)
     assert torch.equal(got, want) and torch.equal(got_res, want_res)
     assert got.float().abs().sum() > 0
 
@@ -268,7 +292,8 @@ def test_packed_gemm_replays_in_a_graph():
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=2)
     pw = pack_weight(b.t())
     scale, one = (sa.view(-1)[:1] * sw.view(-1)[:1]).contiguous(), torch.ones(1, device="cuda")
-    want = skinny_gemm_scaled(a, b, scale, one)
+    with one_plan_for_both_layouts((m, n, k)):
+        want = skinny_gemm_scaled(a, b, scale, one)
     out = torch.empty_like(want)
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
