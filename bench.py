@@ -21,6 +21,10 @@ Other workloads, same method, for the remaining configurations:
   pack        the step before the path: the four Llama-3-8B weights packed into the load format from float8_e4m3fn,
               packed from float8_e4m3fnuz (re-encoded on the way) and unpacked again: 12 launches per step, 2*N*K
               bytes each (`hf_rocm_kernels.utils.weight_format`)
+  floor       what bounds a launch from below, measured with the library's probe kernels: an empty kernel with the GEMM's
+              launch geometry as a graph node, the row-split GEMM's weight requests alone (no activations, no LDS, no matrix
+              instructions, no output) for each of the eight Llama-3 8B / 70B weights, and the same on a 1.9 GB weight for
+              the sustained read rate; `cases` holds the table
 `--packed` runs any of the GEMM/MLP workloads on weights in that load format instead of row-major [N, K].
 
 The calls of a step are captured once into a HIP graph (the reference times its kernel the same way,
@@ -34,8 +38,10 @@ traffic     = HBM bytes per launch read back from rocprofv3 counters (FETCH_SIZE
               script with `--copy-calibration`, which appends a plain 256 MiB device copy whose counter reading
               fixes the scale); the figure is a constant below because a benchmark cannot profile itself
 
-Prints one JSON line.  `--detail` adds a per-(shape, M) table measured outside the timed region, and for the GEMM
-workloads the cache-hot time of each case (one weight copy read over and over).
+Before the timed steps the graphs are replayed for at least 0.3 s (`config.preroll_ms`), so that a short run and a long
+one see the same clocks.  After them every (shape, M) case is timed on its own, outside the timed region (`cases`:
+microseconds per call HBM-cold and cache-hot, GB/s, fraction of peak; `roofline.min_frac_m_le_8` is the smallest fraction
+among the cases with M <= 8); `--no-cases` skips that.  Prints one JSON line.
 """
 import argparse
 import json
@@ -477,13 +483,91 @@ def run_pack_workload(torch, args):
     return result
 
 
+def preroll(torch, graphs, seconds=0.3):
+    """Replay the graphs until `seconds` of wall time have passed; returns the milliseconds it took."""
+    t0 = time.perf_counter()
+    i = 0
+    while True:
+        for _ in range(8):
+            graphs[i % len(graphs)].replay()
+            i += 1
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 >= seconds:
+            return (time.perf_counter() - t0) * 1e3
+
+
+def run_floor_workload(torch, args):
+    """Launch floor, weight-stream-only time per shape and sustained read rate, from the library's probe kernels."""
+    from hf_rocm_kernels import _capi
+    lib = _capi.load()
+    _capi.check(lib.hfrk_init(), "hfrk_init")
+    arena = torch.randint(0, 120, (3 << 30,), dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.Stream()
+
+    def graph_of(calls):
+        with torch.cuda.stream(stream):
+            calls[0]()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for c in calls:
+                c()
+        return g
+
+    def raw():
+        return torch.cuda.current_stream().cuda_stream
+
+    def probe(offset, n, k, grid=256):
+        def call():
+            _capi.check(lib.hfrk_probe_weight_stream(arena.data_ptr() + offset, sink.data_ptr(), n, k, k, grid, raw()), "hfrk_probe_weight_stream")
+        return call
+
+    big_n, big_k = 229376, 8192  # 1.88 GB in one launch
+    big = graph_of([probe(0, big_n, big_k)])
+    pre_ms = preroll(torch, [big])
+    empty = graph_of([lambda: _capi.check(lib.hfrk_probe_empty_launch(raw()), "hfrk_probe_empty_launch")] * 64)
+    empty_us, _ = time_graph(torch, empty, 64, 40)
+    big_us, _ = time_graph(torch, big, 1, 20)
+    sustained = big_n * big_k / big_us / 1e3
+    rows = []
+    for name, n, k in WORKLOADS["llama3-8b"]["shapes"] + WORKLOADS["llama3-70b"]["shapes"]:
+        wbytes = n * k
+        copies = max(3, min(48, arena.numel() // wbytes))
+        g = graph_of([probe(i * wbytes, n, k) for i in range(copies)])
+        us, std = time_graph(torch, g, copies, 40)
+        hot = graph_of([probe(0, n, k)] * 32)
+        us_hot, _ = time_graph(torch, hot, 32, 40)
+        rows.append({"shape": name, "n": n, "k": k, "weight_mb": round(wbytes / 1e6, 2), "stream_only_us": round(us, 3), "us_std": round(std, 3),
+                     "stream_only_gbps": round(wbytes / us / 1e3, 1), "stream_only_frac_of_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                     "stream_only_us_cache_hot": round(us_hot, 3),
+                     "model_us": round(empty_us + wbytes / sustained / 1e3, 3)})
+        del g, hot
+    return {
+        "metric": "launch floor and weight-stream-only time of the FP8 skinny GEMM's own load pattern; value = sustained read rate",
+        "value": round(sustained, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(big_us / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "probe kernels of libhfrk_gfx950.so: hfrk_probe_empty_launch (256 x 512 threads, 64 KB LDS) x 64 in a graph; "
+                               "hfrk_probe_weight_stream on a %d x %d weight (%.2f GB) and on the eight Llama-3 8B / 70B weights, "
+                               "one graph node per weight copy (HBM-cold) and 32 nodes on one copy (cache-hot)" % (big_n, big_k, big_n * big_k / 1e9),
+                   "preroll_ms": round(pre_ms, 1), "timing": "HIP graph replay, HIP events, median of 40"},
+        "roofline": {"bound": "hbm", "achieved": round(sustained, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(sustained / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "hfrk::probe_weight_stream_kernel",
+                     "bytes_per_launch": big_n * big_k, "us_per_launch": round(big_us, 3)},
+        "empty_graph_node_us": round(empty_us, 3),
+        "cases": rows,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "pack"], default="llama3-8b")
-    ap.add_argument("--detail", action="store_true", help="also time every case on its own (HBM-cold and cache-hot)")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "pack", "floor"], default="llama3-8b")
+    ap.add_argument("--detail", action="store_true", help="kept for older command lines: the per-case table is on by default")
+    ap.add_argument("--no-cases", action="store_true", help="skip the per-case table after the timed steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--packed", action="store_true",
                     help="weights in the library's packed load format (hfrk_pack_weight) instead of row-major [N, K]")
@@ -500,6 +584,9 @@ def main():
 
     if args.workload == "pack":
         print(json.dumps(run_pack_workload(torch, args)))
+        return
+    if args.workload == "floor":
+        print(json.dumps(run_floor_workload(torch, args)))
         return
     is_mlp = args.workload in ("mlp", "mlp-fused")
     if is_mlp:
@@ -525,6 +612,7 @@ def main():
         n_copies = len(spec["ms"]) * spec["cycle"]
     cycle = len(graphs)
 
+    preroll_ms = preroll(torch, graphs)
     for i in range(args.warmup):
         graphs[i % cycle].replay()
     torch.cuda.synchronize()
@@ -556,7 +644,7 @@ def main():
         "config": {"workload": text, "calls_per_step": calls, "bytes_per_step": step_bytes,
                    "weight_copies_per_shape": n_copies,
                    "weight_layout": "packed 16x256-byte chunks in MFMA operand order (hfrk_pack_weight)" if args.packed else "row-major [N, K]",
-                   "timing": "HIP graph replay, HIP events",
+                   "timing": "HIP graph replay, HIP events", "preroll_ms": round(preroll_ms, 1),
                    "plan_table": os.environ.get("HFRK_PLAN_TABLE", "shipped (hf_rocm_kernels/plan_tables/gfx950_*.json)"),
                    "us_per_call_mean": round(ms_per_step * 1e3 / calls, 3), "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -574,11 +662,15 @@ def main():
         torch.cuda.synchronize()
         result["config"]["calibration_copy_bytes"] = CALIBRATION_COPY_BYTES
         del src, dst
-    if args.detail:
+    if not args.no_cases:
         if is_mlp:
             result["cases"] = time_mlp_cases(torch, call)
         else:
             result["cases"] = time_gemm_cases(torch, spec, call, weights)
+            small = [c["frac_of_peak"] for c in result["cases"] if c["m"] <= 8]
+            if small:
+                result["roofline"]["min_frac_m_le_8"] = min(small)
+                result["roofline"]["mean_frac_m_le_8"] = round(sum(small) / len(small), 4)
     del graphs, keep, call
     if is_mlp:
         del copies, acts

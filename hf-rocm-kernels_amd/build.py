@@ -24,7 +24,7 @@ INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["hfrk_common.hip", "skinny_gemm.hip", "skinny_gemm_stream.hip", "skinny_gemm_rows.hip", "skinny_gemm_ksplit.hip", "residual_rms.hip", "swiglu.hip",
-               "dynamic_quant.hip", "pack_weight.hip", "plan_table_file.hip"]
+               "dynamic_quant.hip", "pack_weight.hip", "plan_table_file.hip", "probe.hip"]
 LIB_NAME = "libhfrk_gfx950.so"
 EXT_NAME = "_HFRK_C.abi3.so"
 

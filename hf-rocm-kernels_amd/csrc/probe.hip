@@ -1,0 +1,112 @@
+// Measurement probes: what a launch costs before it does anything, and what the GEMM's own weight requests cost when
+// nothing is computed.  They give the floor the skinny-GEMM kernels are measured against (launch + first-byte latency +
+// bytes / sustained bandwidth), per weight shape.  No counterpart in the reference, which publishes timings only
+// (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:45-88).
+#include "skinny_gemm_args.h"
+
+namespace hfrk {
+
+// A kernel with the GEMM's launch geometry (256 workgroups x 512 threads, 64 KB of LDS) that does nothing.
+__global__ void __launch_bounds__(kGemmThreads) probe_empty_kernel(int* sink) {
+    if (sink == reinterpret_cast<int*>(1)) sink[0] = 0;
+}
+
+// The row-split kernel's weight requests and nothing else: the same bands of rows per workgroup, the same tiles, the same
+// runs of 16-row x 256-byte chunks per wave, four 16-byte `nt` loads per lane and chunk (4 rows x 256 contiguous bytes per
+// instruction), one chunk in flight per wave.  The loaded registers are folded into one value so that every load is
+// waited for; the value is stored only if it has a bit pattern that the fold of any data cannot produce twice in a row.
+__global__ void __launch_bounds__(kGemmThreads) probe_weight_stream_kernel(const GemmArgs a) {
+    constexpr uint32_t kOutOfRange = 0x80000000u;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int G = a.grid;
+    const int b = blockIdx.x;
+    const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;
+    const bool tall = g < a.rows_r;
+    const int u0 = g * a.rows_q + min(g, a.rows_r);
+    const int T = tall ? a.tiles_a : a.tiles_b;
+    const int ubase = tall ? a.base_a : a.base_b;
+    const int uextra = tall ? a.extra_a : a.extra_b;
+    const int KC = a.slabs;
+    const int TC = T * KC;
+    const int i0 = (wv * TC) >> 3, i1 = ((wv + 1) * TC) >> 3;
+    const int count = i1 - i0;
+    int itile = (int)__umulhi((uint32_t)i0, a.kc_magic);
+    int ikc = i0 - itile * KC;
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
+    const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
+    int iunits = ubase + (itile < uextra ? 1 : 0);
+    int irow0 = 4 * (u0 + itile * ubase + min(itile, uextra));
+    uint32_t irow_off = (uint32_t)irow0 * (uint32_t)a.b_stride;
+    v4i wq[4];
+    auto issue_chunk = [&]() __attribute__((always_inline)) {
+        const uint32_t kbyte = (uint32_t)ikc * 256u;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t off = t < iunits ? irow_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.b_stride : kOutOfRange;
+            wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + off), 0, 2 /* nt */);
+        }
+    };
+    if (count > 0) issue_chunk();
+    v4i fold = {0, 0, 0, 0};
+    for (int i = 0; i < count; ++i) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) fold ^= wq[t];
+        if (i + 1 < count) {
+            if (++ikc == KC) {
+                ikc = 0;
+                irow0 += 4 * iunits;
+                irow_off = (uint32_t)irow0 * (uint32_t)a.b_stride;
+                ++itile;
+                iunits = ubase + (itile < uextra ? 1 : 0);
+            }
+            issue_chunk();
+        }
+    }
+    if (fold[0] == 0x12345678 && fold[1] == (int)0x9abcdef0 && fold[2] == 0x0fedcba9 && fold[3] == 0x87654321)
+        reinterpret_cast<int*>(a.D)[0] = fold[0];
+}
+
+}  // namespace hfrk
+
+extern "C" {
+
+int hfrk_probe_empty_launch(void* stream) {
+    static int* sink = nullptr;  // never dereferenced by the kernel
+    hipLaunchKernelGGL(hfrk::probe_empty_kernel, dim3(hfrk::kNumCU), dim3(hfrk::kGemmThreads), 64 * 1024, static_cast<hipStream_t>(stream), sink);
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}
+
+int hfrk_probe_weight_stream(const void* B, void* sink, int n, int k, int b_stride, int grid, void* stream) {
+    if (!B || !sink || n < 1 || k < 512 || k % 256 != 0 || b_stride < k || (b_stride & 15) || (reinterpret_cast<uintptr_t>(B) & 15))
+        return HFRK_BAD_SHAPE;
+    if (((long)n + 128) * b_stride + k >= (1L << 31)) return HFRK_BAD_SHAPE;
+    const int units = (n + 3) / 4;
+    if (grid < 1 || grid > hfrk::kMaxGrid || grid > units) return HFRK_INVALID_CONFIG;
+    hfrk::GemmArgs args = {};
+    args.B = static_cast<const uint8_t*>(B);
+    args.D = sink;
+    args.n = n;
+    args.k = k;
+    args.b_stride = b_stride;
+    args.grid = grid;
+    args.slabs = k / 256;
+    args.rows_q = units / grid;
+    args.rows_r = units % grid;
+    auto geometry = [](int u, int* tiles, int* base, int* extra) {
+        *tiles = (u + 3) / 4;
+        *base = *tiles ? u / *tiles : 0;
+        *extra = *tiles ? u % *tiles : 0;
+    };
+    geometry(args.rows_q + 1, &args.tiles_a, &args.base_a, &args.extra_a);
+    geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
+    args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)args.slabs - 1) / (uint64_t)args.slabs);
+    hipLaunchKernelGGL(hfrk::probe_weight_stream_kernel, dim3(grid), dim3(hfrk::kGemmThreads), 0, static_cast<hipStream_t>(stream), args);
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
+}
+
+}  // extern "C"

@@ -170,6 +170,68 @@ def test_llama_mlp_chain(m, add_residual, fused):
     assert float(dl.mean()) < 0.03 * float(loose_out.float().std()) + 1e-2
 
 
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("add_residual", [False, True])
+@pytest.mark.parametrize("m", [1, 8, 16])
+def test_llama_mlp_chain_stage_by_stage(m, add_residual, fused):
+    """BASELINE config 4 held to the strict bar, one stage at a time: every stage of the device chain is compared with the
+    oracle's next stage fed with the device's own output of the stage before (so that an fp8 boundary flip upstream cannot
+    move the comparison), and the block's result must be, bit for bit, what these stages give when run one by one.
+    Order of the chain: hf_rocm_kernels/combined_ops/llama_mlp.py:23-59 of the reference."""
+    from hf_rocm_kernels import residual_rms, skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu, swiglu
+    from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
+    from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
+    from oracle import residual_rms as orms
+    from oracle import swiglu as osw
+    from test_gemm_gpu import _swiglu_oracle, check_against_oracle
+    hidden, inter = 4096, 14336
+    g = torch.Generator().manual_seed(20 + m)
+    dtype = torch.bfloat16
+    attn = torch.randn(m, hidden, generator=g).to(dtype)
+    resid = torch.randn(m, hidden, generator=g).to(dtype)
+    rms_w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    wgu = torch.randn(2 * inter, hidden, generator=g) * 0.02
+    wd = torch.randn(hidden, inter, generator=g) * 0.02
+    s_gu, s_d = amax_scale(wgu), amax_scale(wd)
+    wgu8, wd8 = fp8_quantize(wgu, s_gu)[0].cuda().t(), fp8_quantize(wd, s_d)[0].cuda().t()
+    in_gu = torch.tensor([6.0 / 448], dtype=torch.float32).cuda()
+    in_d = torch.tensor([4.0 / 448], dtype=torch.float32).cuda()
+    out_gu, out_d = (in_gu * s_gu.cuda()).reshape(1), (in_d * s_d.cuda()).reshape(1)
+    one = torch.ones(1).cuda()
+    block_out, block_res = llama_mlp_combined_ops(attn.cuda(), resid.cuda(), rms_w.cuda(), 1e-5, wgu8, in_gu, out_gu, wd8, in_d, out_d,
+                                                  add_residual=add_residual, fused=fused)
+
+    # 1. residual RMSNorm -> fp8: the residual bit for bit, the fp8 values within one step of the float64 result, rarely off
+    normalized, res = residual_rms(attn.cuda(), resid.cuda(), rms_w.cuda(), 1e-5, scale_tensor=in_gu)
+    want_res = (attn.float() + resid.float()).to(dtype)
+    assert torch.equal(res.cpu().view(torch.int16), want_res.view(torch.int16)) and torch.equal(res, block_res)
+    q_ref, _ = orms.precise_residual_rms(want_res, torch.zeros_like(want_res), rms_w, 1e-5, in_gu.cpu())
+    d = (normalized.cpu().float() - q_ref.float()).abs()
+    assert (d <= torch.maximum(q_ref.float().abs() * 2.0 ** -3, torch.tensor(2.0 ** -9))).all() and (d > 0).float().mean() < 0.01
+
+    # 2 + 3. gate_up projection and SwiGLU of the device's own normalised activations
+    if fused:
+        act = skinny_gemm_swiglu(normalized, wgu8, out_gu, None, in_d, intermediate_dtype=dtype)
+        ref, tol = _swiglu_oracle(normalized, wgu8, out_gu, one, in_d, dtype)
+        d = (act.cpu().float() - ref.float()).abs()
+        assert (d <= tol).all() and (d > 0).float().mean() < 0.02
+    else:
+        gate_up = skinny_gemm(normalized, wgu8, out_gu, torch.zeros((m, 2 * inter), dtype=dtype, device="cuda"))
+        check_against_oracle(gate_up, normalized, wgu8, out_gu, one)      # exact-product bound and rtol/atol 1e-2, every element
+        act = swiglu(gate_up, in_d)
+        ref = osw.reference_swiglu(gate_up.cpu(), in_d.cpu())
+        d = (act.cpu().float() - ref.float()).abs()
+        assert (d <= torch.maximum(ref.float().abs() * 2.0 ** -3, torch.tensor(2.0 ** -9))).all() and (d > 0).float().mean() < 0.01
+
+    # 4. down projection (+ residual) of the device's own fp8 activations: every element within the bound and rtol/atol 1e-2
+    if add_residual:
+        out = skinny_gemm_add(act, wd8, out_d, None, base=res)
+    else:
+        out = skinny_gemm_scaled(act, wd8, out_d, one)
+    check_against_oracle(out, act, wd8, out_d, one, base=res if add_residual else None)
+    assert torch.equal(out, block_out), "the block is not the chain of its stages"
+
+
 # ---- per-row dynamic quantisation ----------------------------------------------------------------------------------------
 
 def _check_dynamic(q_dev, scales_dev, q_ref, scales_ref, y):
