@@ -638,18 +638,34 @@ static int fill_rows_plan(int m, int n, int k, int row_tiles, int grid_hint, hfr
     return HFRK_SUCCESS;
 }
 
-// The planner takes the row-split decomposition when the 4-row units deal out evenly: at least one per workgroup and the
-// busiest workgroup at most a tenth above the mean (on 2304 x 16384, 2.25 units per workgroup, splitting K between
-// workgroups is the better cut).  Two matrix tiles per chunk from 9 rows on, once a band has 24 rows to fill them
-// (57344 x 8192 at 16 rows: 72.3 against 79.5 us; 4096 x 4096, 16 rows per band: 5.7 against 6.3 the other way).
+// The planner takes the row-split decomposition when there is at least one 4-row unit per workgroup and the busiest
+// workgroup is at most 40 % above the mean (2304 x 16384, 2.25 units per workgroup: 9.5 us against 10.3 for the wave-stream
+// split).  Sweeps over 23 weight shapes say what else matters:
+//  * tiles that are not full (a band height that is no multiple of 16 rows) cost 3-11 %, because a wave keeps one chunk
+//    in flight and a 12-row chunk is 3 KB instead of 4.  So a grid between 224 and 256 that gives every workgroup whole
+//    16-row tiles is taken when there is one (3584 rows: 224 workgroups, 4.6 against 5.2 us); otherwise, up to 4
+//    activation rows and bands of at most 48 rows, twice the workgroups with half the band each put more bytes in flight
+//    (6144 x 4096: 6.05 against 6.5 us; 10240 x 8192: 14.9 against 15.6; no gain from 5 rows on, where the activation
+//    loads of 16 waves per CU weigh in);
+//  * two matrix tiles per chunk from 9 rows on, once a band has 24 rows to fill them (57344 x 8192 at 16 rows: 72.3
+//    against 79.5 us; 4096 x 4096, 16 rows per band: 5.7 against 6.3 the other way).
 static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m > kRowsMaxM || k < 512) return HFRK_INVALID_CONFIG;
     const long units = (n + 3) / 4;
     if (units < kNumCU) return HFRK_INVALID_CONFIG;
-    const long busiest = (units + kNumCU - 1) / kNumCU;
-    if (units * 10 < busiest * kNumCU * 9) return HFRK_INVALID_CONFIG;
-    const int row_tiles = (m >= 9 && 4 * busiest >= 24) ? 2 : 1;
-    return fill_rows_plan(m, n, k, row_tiles, 0, plan);
+    long grid = kNumCU;
+    const long busiest = (units + grid - 1) / grid;
+    if (units * 10 < busiest * grid * 7) return HFRK_INVALID_CONFIG;
+    if (units % (4 * grid) != 0) {
+        long whole = 0;
+        for (long g = kNumCU - 8; g >= 7 * kNumCU / 8; g -= 8)
+            if (units % (4 * g) == 0) { whole = g; break; }
+        if (whole) grid = whole;
+        else if (m <= 4 && 4 * busiest <= 48 && units >= 4 * kNumCU) grid = 2 * kNumCU;  // bands of at least 8 rows
+    }
+    const long rows_per_band = 4 * ((units + grid - 1) / grid);
+    const int row_tiles = (m >= 9 && rows_per_band >= 24) ? 2 : 1;
+    return fill_rows_plan(m, n, k, row_tiles, (int)grid, plan);
 }
 
 // 17 <= m <= 64 (valid from 1): the waves of a workgroup split K windows of 8*wave_k bytes, activations in registers
@@ -746,15 +762,16 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
 }
 
 static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p, bool packed = false) {
-    if (swiglu && p->wn != 0) return HFRK_INVALID_CONFIG;  // the fused epilogue exists in the wave-stream kernel only
+    if (swiglu && p->wn != 0 && p->wn != -2) return HFRK_INVALID_CONFIG;  // the fused epilogue: wave-stream and row-split kernels
     if (p->wn == -2) {  // row-split decomposition: wk = matrix tiles per chunk, ch = activation loads
-        if (packed || swiglu) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
+        if (packed) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
+        if (swiglu && p->wk != 2) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows
         if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
         if (p->m_tiles != 1 || p->panels != (n + 3) / 4 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
         if (p->lds_bytes != rows_lds_bytes(p->wk)) return HFRK_INVALID_CONFIG;
         // a band's chunk indices stay far below 2^32 / slabs (the kernel divides by multiplying with a reciprocal)
-        if (((long)p->panels / p->grid / (4 * p->wk) + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;
+        if (((long)p->panels / p->grid / 4 + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;
         return HFRK_SUCCESS;
     }
     if (p->wn == -1) {  // K-split decomposition: wk = wave_k / 256
@@ -906,12 +923,20 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         const int rc = check_plan(m, swiglu ? n / 2 : n, k, swiglu, &p, packed);
         if (rc != HFRK_SUCCESS) return rc;
     } else {
-        const int rc = swiglu ? fill_stream_plan(m, n / 2, k, 1, false, 0, &p) : choose_plan(m, n, k, packed, &p);
-        if (rc != HFRK_SUCCESS) return rc;
-        if (swiglu) {  // same chunk count as a one-tile plan over n/2 rows, but every chunk holds a gate and an up tile
-            p.wk = 2;
-            p.lds_bytes = stream_lds_bytes(p.ch, 2);
+        int rc;
+        if (swiglu && !packed && make_rows_plan(m, n / 2, k, &p) == HFRK_SUCCESS) {
+            // bands of output columns; every chunk holds the gate rows and the up rows of up to 16 of them
+            rc = fill_rows_plan(m, n / 2, k, 2, p.grid, &p);
+        } else if (swiglu) {
+            rc = fill_stream_plan(m, n / 2, k, 1, false, 0, &p);
+            if (rc == HFRK_SUCCESS) {  // the chunk count of a one-tile plan over n/2 rows, but every chunk holds a gate and an up tile
+                p.wk = 2;
+                p.lds_bytes = stream_lds_bytes(p.ch, 2);
+            }
+        } else {
+            rc = choose_plan(m, n, k, packed, &p);
         }
+        if (rc != HFRK_SUCCESS) return rc;
     }
 
     int dev = 0;
@@ -969,7 +994,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     args.ws_bytes = (uint32_t)ws_bytes;
     args.counters = st.counters;
     if (p.wn == -2) {
-        const int per_tile = 4 * p.wk;  // units a tile can hold
+        const int per_tile = swiglu ? 4 : 4 * p.wk;  // units a tile can hold (SwiGLU: 16 output columns, their gate and their up rows)
         args.rows_q = p.panels / p.grid;
         args.rows_r = p.panels % p.grid;
         auto geometry = [&](int units, int* tiles, int* base, int* extra) {
@@ -980,7 +1005,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         geometry(args.rows_q + 1, &args.tiles_a, &args.base_a, &args.extra_a);
         geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
         args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)p.slabs - 1) / (uint64_t)p.slabs);
-        return launch_rows_kernel(args, p.ch, p.wk, p.lds_bytes, stream);
+        return launch_rows_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     }
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, p.lds_bytes, stream);

@@ -55,7 +55,9 @@ constexpr bool stream_variant_exists(int act_loads, int row_tiles, bool swiglu =
 
 // row-split wave-stream kernel (m <= 16), skinny_gemm_rows.hip: every workgroup owns a band of weight rows and all of k;
 // act_loads = ceil(m/4), row_tiles = 16-row matrix tiles per chunk (1 or 2).  Needs k >= 512.
-int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream);
+// swiglu: gate rows [0, n/2), up rows [n/2, n); row_tiles must be 2 (a gate and an up tile per chunk), bands and tiles count
+// the n/2 output columns, D is fp8 [m, n/2]
+int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream);
 constexpr int kRowsMaxM = 16;
 constexpr int rows_lds_bytes(int row_tiles) { return kGemmWaves * (row_tiles + 1) * kTileBytes; }
 constexpr bool rows_variant_exists(int act_loads, int row_tiles) {

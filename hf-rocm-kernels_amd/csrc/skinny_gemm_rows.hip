@@ -39,8 +39,13 @@ __device__ __forceinline__ uint32_t pack16(float lo, float hi, bool bf16) {
 }
 
 // MA = ceil(m/4): 16-byte activation loads per lane and chunk (rows 4t .. 4t+3), RT = 16-row matrix tiles per chunk.
-template <int MA, int RT>
+// SWIGLU: the weight is a gate_up projection (gate rows [0, n/2), up rows [n/2, n)).  Bands, units and tiles then count
+// output columns (n/2 of them); a chunk pairs up to 16 gate rows with the up rows of the same columns (RT = 2: the gate
+// tile and the up tile), and the epilogue stores e4m3fn(silu(gate) * up / out_scale) into D [m, n/2] instead of the two
+// 16-bit projections -- the SwiGLU kernel of csrc/op_src/swiglu/swiglu_vectorized.cu:27-97 as the GEMM's epilogue.
+template <int MA, int RT, bool SWIGLU>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const GemmArgs a) {
+    static_assert(!SWIGLU || RT == 2, "the SwiGLU epilogue pairs one gate tile with one up tile");
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kWaveLds = (RT + 1) * kTileBytes;  // RT weight tiles, one activation tile
     constexpr int kSlotStride = kWaveLds / 16;       // in v4f
@@ -87,7 +92,10 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
             aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
 #pragma unroll
         for (int t = 0; t < 4 * RT; ++t) {  // unit t of the tile; a unit the tile does not have reads as zero, without traffic
-            const uint32_t off = t < iunits ? irow_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.b_stride : kOutOfRange;
+            // SWIGLU: loads 0..3 fetch the tile's gate rows, loads 4..7 the up rows of the same columns, n/2 rows further down
+            const int unit = SWIGLU ? t % 4 : t;
+            const uint32_t row = SWIGLU ? (uint32_t)(4 * unit + (t / 4) * (a.n >> 1)) : (uint32_t)(4 * t);
+            const uint32_t off = unit < iunits ? irow_off + kbyte + row * (uint32_t)a.b_stride : kOutOfRange;
             wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + off), 0, 2 /* nt */);
         }
     };
@@ -104,15 +112,21 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     __builtin_amdgcn_sched_barrier(0);  // keep the set-up below behind the first request
 
     // ---- the rest of the set-up, while the first chunk is on its way -------------------------------------------------
-    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
+    const int n_out = SWIGLU ? (a.n >> 1) : a.n;  // columns of D
+    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)n_out * (SWIGLU ? 1u : 2u));
     const __amdgpu_buffer_rsrc_t base_rsrc = make_rsrc(a.base, a.base ? (uint32_t)a.m * (uint32_t)a.n * 2u : 0u);
     const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
-    const bool accumulate = a.base != nullptr;
-    const bool vec = (a.n & 3) == 0;  // then a lane's four outputs are all inside n and 8-byte aligned
+    const bool accumulate = !SWIGLU && a.base != nullptr;
+    const bool vec = SWIGLU || (a.n & 3) == 0;  // then a lane's four outputs are all inside n and aligned
     const bool per_channel = a.scale_b && a.sb_stride;
     const bool bf16 = a.d_dtype == HFRK_BF16;
     // lane li holds the accumulator column of activation row li
     const float sa = a.scale_a[(long)min(li, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+    float inv_out_scale = 1.0f;
+    if constexpr (SWIGLU) {
+        const float os = a.out_scale[0];
+        inv_out_scale = os != 0.f ? 1.0f / os : 1.0f;
+    }
 
     uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its activation tile
     uint8_t* const ta = tw + RT * kTileBytes;
@@ -140,8 +154,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
         if (wanted && want_pre) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                const int ul = 4 * rt + lg;  // this lane's unit of the tile
-                const int n0 = row0 + 4 * ul;
+                const int ul = SWIGLU ? lg : 4 * rt + lg;                        // this lane's unit of the tile
+                const int n0 = row0 + 4 * ul + (SWIGLU ? rt * (a.n >> 1) : 0);  // its first weight row (= scale channel)
                 const bool ok = ul < units && n0 < a.n;
                 p.sb[rt] = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (per_channel && ok) ? n0 * 4 : (int)kOutOfRange, 0, 0);
                 p.d[rt] = __builtin_amdgcn_raw_buffer_load_b64(base_rsrc, (accumulate && ok && li < a.m) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
@@ -152,6 +166,26 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
 
     // scale, add D (accumulate mode), round once, store: lane holds D[li][n0 + v], v = 0..3, n0 = row0 + 16*rt + 4*lg
     auto epilogue = [&](int row0, int units, const v4f (&acc)[RT], const Pre& pre) __attribute__((always_inline)) {
+        if constexpr (SWIGLU) {
+            // acc[0] = gate, acc[1] = up of output columns n0 .. n0+3.  The unfused chain stores both projections in the
+            // 16-bit dtype between its two kernels: round them the same way before the activation.
+            const int n0 = row0 + 4 * lg;
+            const v4f sbg = __builtin_bit_cast(v4f, pre.sb[0]), sbu = __builtin_bit_cast(v4f, pre.sb[RT - 1]);
+            float y[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float g = acc[0][v] * (sa * (per_channel ? sbg[v] : 1.0f));
+                float u = acc[RT - 1][v] * (sa * (per_channel ? sbu[v] : 1.0f));
+                g = bf16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(g)) : load16<HFRK_F16>(store16<HFRK_F16>(g));
+                u = bf16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(u)) : load16<HFRK_F16>(store16<HFRK_F16>(u));
+                y[v] = silu_mul(g, u, inv_out_scale);
+            }
+            uint32_t packed = cvt_pk_fp8(y[0], y[1], 0u, false);
+            packed = cvt_pk_fp8(y[2], y[3], packed, true);
+            const bool live = li < a.m && lg < units && n0 < n_out;
+            __builtin_amdgcn_raw_buffer_store_b32((int)packed, d_rsrc, live ? (int)((uint32_t)li * (uint32_t)n_out + (uint32_t)n0) : (int)kOutOfRange, 0, 0);
+            return;
+        }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             const int ul = 4 * rt + lg;
@@ -298,9 +332,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     epilogue(row0_l, units_l, acc, pre_l);
 }
 
-template <int MA, int RT>
+template <int MA, int RT, bool SWIGLU>
 static int launch_rows_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_rows_kernel<MA, RT>;
+    auto kern = skinny_gemm_rows_kernel<MA, RT, SWIGLU>;
     static bool attr_done[kMaxDevices] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -313,12 +347,14 @@ static int launch_rows_one(const GemmArgs& args, int lds_bytes, hipStream_t stre
     return HFRK_SUCCESS;
 }
 
-int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, int lds_bytes, hipStream_t stream) {
+int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream) {
     if (!rows_variant_exists(act_loads, row_tiles) || lds_bytes != rows_lds_bytes(row_tiles)) return HFRK_INVALID_CONFIG;
-#define HFRK_ROWS_CASE(MA_)                                                                \
-    case MA_:                                                                              \
-        return row_tiles == 1 ? launch_rows_one<MA_, 1>(args, lds_bytes, stream)           \
-                              : launch_rows_one<MA_, 2>(args, lds_bytes, stream);
+    if (swiglu && row_tiles != 2) return HFRK_INVALID_CONFIG;
+#define HFRK_ROWS_CASE(MA_)                                                                     \
+    case MA_:                                                                                   \
+        if (swiglu) return launch_rows_one<MA_, 2, true>(args, lds_bytes, stream);              \
+        return row_tiles == 1 ? launch_rows_one<MA_, 1, false>(args, lds_bytes, stream)         \
+                              : launch_rows_one<MA_, 2, false>(args, lds_bytes, stream);
     switch (act_loads) {
         HFRK_ROWS_CASE(1)
         HFRK_ROWS_CASE(2)

@@ -375,6 +375,25 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
         f = out.cpu().float()
         assert not f.isnan().any(), grid
         assert ((f - ref.float()).abs() <= tol).all(), grid
+    if k < 512:
+        return
+    # row-split plans: bands of output columns, cut between waves inside a workgroup only
+    units = (n // 2 + 3) // 4
+    for grid in sorted({min(g, units) for g in (512, 256, 224, 200, 64, 7, 1)}):
+        plan = _capi.GemmPlan(1, -2, 2, ma, grid, units, kc, 8 * 3 * 4096)
+        out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
+        st = lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                                        out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
+                                        ctypes.byref(plan), torch.cuda.current_stream().cuda_stream)
+        assert st == 0, ("rows", grid, st)
+        torch.cuda.synchronize()
+        f = out.cpu().float()
+        assert not f.isnan().any(), ("rows", grid)
+        assert ((f - ref.float()).abs() <= tol).all(), ("rows", grid)
+    one_tile = _capi.GemmPlan(1, -2, 1, ma, 64, units, kc, 8 * 2 * 4096)  # a chunk must hold a gate and an up tile
+    assert lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                                      out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
+                                      ctypes.byref(one_tile), torch.cuda.current_stream().cuda_stream) == _capi.INVALID_CONFIG
 
 
 def test_benchmarking_helpers_and_the_library_gemm_agree_with_scaled_mm():

@@ -183,7 +183,7 @@ def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
     plan = _capi.plan(m, n, k)
     if plan.wn == -2:  # m <= 16, rows that deal out evenly: row-split decomposition
         assert m <= 16 and plan.ch == (m + 3) // 4 and plan.m_tiles == 1 and plan.slabs == k // 256 and plan.panels == -(-n // 4)
-        assert plan.wk in (1, 2) and plan.lds_bytes == 8 * (plan.wk + 1) * 4096 and 1 <= plan.grid <= min(256, plan.panels)
+        assert plan.wk in (1, 2) and plan.lds_bytes == 8 * (plan.wk + 1) * 4096 and 1 <= plan.grid <= min(512, plan.panels)
         _emulate_rows(plan)
         return
     if plan.wn == 0:  # m <= 16: wave-stream decomposition
