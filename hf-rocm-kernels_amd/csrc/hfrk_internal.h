@@ -64,7 +64,10 @@ __device__ __forceinline__ uint16_t store16(float f) {
 }
 
 // ---- fp32 -> OCP e4m3fn, saturating to +-448, round to nearest even ------------------------------------------
-// v_cvt_pk_fp8_f32 on gfx950 produces OCP e4m3fn; the clamp makes the saturation explicit (NaN stays NaN).
+// v_cvt_pk_fp8_f32 on gfx950 produces OCP e4m3fn; the clamp makes the saturation explicit.  A NaN does not survive the
+// clamp: v_med3_f32 with a NaN operand returns the minimum of the other two, so NaN is stored as -448 (0xFE), which is
+// also what the reference's clamp-then-convert does with it.  The CPU oracle's encoder maps NaN to 0x7F instead; the two
+// meet only on inputs that are already invalid.
 __device__ __forceinline__ uint32_t cvt_pk_fp8(float a, float b, uint32_t old, bool high) {
     a = __builtin_amdgcn_fmed3f(a, 448.0f, -448.0f);
     b = __builtin_amdgcn_fmed3f(b, 448.0f, -448.0f);

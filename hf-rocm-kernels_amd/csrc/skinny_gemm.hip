@@ -570,7 +570,7 @@ static int fill_stream_plan(int m, int n, int k, int row_tiles, bool swiglu, int
     if (!stream_variant_exists(act_loads, row_tiles, swiglu)) return HFRK_INVALID_CONFIG;
     const long tiles = (n + 16 * row_tiles - 1) / (16 * row_tiles);  // swiglu: n/2 output columns in tiles of 16
     if (tiles > kMaxPanels) return HFRK_BAD_SHAPE;
-    const int kc = k / 256;
+    const int kc = (k + 255) / 256;  // the last chunk of a row may be cut short (row-major weights, k % 16 == 0)
     const long chunks = tiles * kc;
     long grid = grid_hint > 0 ? grid_hint : kNumCU;
     if (grid > chunks) grid = chunks;
@@ -612,7 +612,7 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (act_loads > 4) {
         row_tiles = 2;
     } else if (act_loads >= 3 && k >= 4096) {
-        const long chunks2 = (long)((n + 31) / 32) * (k / 256);
+        const long chunks2 = (long)((n + 31) / 32) * ((k + 255) / 256);
         if (chunks2 >= (long)kStreamRt2MinChunksPerWave * kNumCU * kGemmWaves) row_tiles = 2;
     }
     return fill_stream_plan(m, n, k, row_tiles, false, 0, plan);
@@ -622,7 +622,7 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 // plan: wn = -2, wk = matrix tiles per chunk, ch = activation loads, panels = 4-row units, slabs = k / 256.
 static int fill_rows_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk_gemm_plan* plan) {
     const int act_loads = (m + 3) / 4;
-    if (m > kRowsMaxM || !rows_variant_exists(act_loads, row_tiles) || k < 512) return HFRK_INVALID_CONFIG;
+    if (m > kRowsMaxM || !rows_variant_exists(act_loads, row_tiles) || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
     const long units = (n + 3) / 4;
     long grid = grid_hint > 0 ? grid_hint : kNumCU;
     if (grid > units) grid = units;
@@ -650,7 +650,7 @@ static int fill_rows_plan(int m, int n, int k, int row_tiles, int grid_hint, hfr
 //  * two matrix tiles per chunk from 9 rows on, once a band has 24 rows to fill them (57344 x 8192 at 16 rows: 72.3
 //    against 79.5 us; 4096 x 4096, 16 rows per band: 5.7 against 6.3 the other way).
 static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
-    if (m > kRowsMaxM || k < 512) return HFRK_INVALID_CONFIG;
+    if (m > kRowsMaxM || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
     const long units = (n + 3) / 4;
     if (units < kNumCU) return HFRK_INVALID_CONFIG;
     long grid = kNumCU;
@@ -732,7 +732,13 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
 
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = false) {
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1) return HFRK_BAD_SHAPE;
-    if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (k % 16 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (k % 256 != 0) {
+        // A row that ends inside a 256-byte chunk: a variant of the wave-stream kernel masks the missing pieces (row-major
+        // weights, up to 32 activation rows; a call with more rows runs as two launches, see gemm_launch).
+        if (packed || m > kStreamMaxM) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+        return make_stream_plan(m, n, k, plan);
+    }
     // k = 1024 is four chunks per row tile: too few for the wave-stream split and half a K-split window.  Four K waves
     // cover it in one slab, so nothing is exchanged between workgroups (1024 x 1024: 4.2 against 5.2 us at 1 row,
     // 5120 x 1024: 5.7 against 7.3 at 32 rows); on weights wider than 12288 rows the other kernels catch up.
@@ -767,6 +773,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
         if (packed) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
         if (swiglu && p->wk != 2) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows
         if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
+        if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
         if (p->m_tiles != 1 || p->panels != (n + 3) / 4 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
         if (p->lds_bytes != rows_lds_bytes(p->wk)) return HFRK_INVALID_CONFIG;
@@ -774,6 +781,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
         if (((long)p->panels / p->grid / 4 + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;
         return HFRK_SUCCESS;
     }
+    if (k % 256 != 0 && (packed || p->wn != 0)) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;  // only the wave-stream kernel cuts a chunk short
     if (p->wn == -1) {  // K-split decomposition: wk = wave_k / 256
         hfrk_gemm_plan want;
         const int rc = fill_ksplit_plan(m, n, k, p->wk * 256, p->grid, &want);
@@ -789,7 +797,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
         if (m > kStreamMaxM || !stream_variant_exists(p->ch, p->wk, swiglu) || 4 * p->ch < m) return HFRK_INVALID_CONFIG;
         if (p->m_tiles != (p->ch + 3) / 4) return HFRK_INVALID_CONFIG;
         const int rows = swiglu ? 16 : 16 * p->wk;  // with the SwiGLU epilogue n counts output columns: one gate + one up tile
-        if (p->panels != (n + rows - 1) / rows || p->slabs != k / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
+        if (p->panels != (n + rows - 1) / rows || p->slabs != (k + 255) / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
         const long chunks = (long)p->panels * p->slabs;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
         if (chunks * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's chunk arithmetic is 32-bit
@@ -899,7 +907,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
                        bool use_static = false) {
     if (packed) b_stride = k;
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
-    if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (k % 16 != 0 || (packed && k % 256 != 0)) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (d_dtype != HFRK_F16 && d_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
     if (!A || !B || !D || !scale_a) return HFRK_BAD_SHAPE;
     if ((sa_stride != 0 && sa_stride != 1) || (sb_stride != 0 && sb_stride != 1)) return HFRK_BAD_SHAPE;
@@ -917,6 +925,20 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         if ((both & 1) || ((n & 3) == 0 && (both & 7))) return HFRK_BAD_ALIGNMENT;
     }
 
+    if (!user_plan && k % 256 != 0 && m > kStreamMaxM) {
+        // A cut-short last chunk is handled by the kernels for up to 32 rows: more rows run as two launches over the
+        // same weight (the reference accepts such k only with its narrowest tiles, skinny_gemm_caller.cu:33-48; the
+        // shapes it is tuned for are all multiples of 256).
+        const int first = kStreamMaxM;
+        const size_t row_bytes = (size_t)n * 2;
+        int rc = gemm_launch(A, B, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, first, n, k, b_stride, d_dtype,
+                             epilogue, nullptr, stream, packed, use_static);
+        if (rc != HFRK_SUCCESS) return rc;
+        return gemm_launch(static_cast<const uint8_t*>(A) + (size_t)first * k, B, static_cast<uint8_t*>(D) + first * row_bytes,
+                           base ? static_cast<const uint8_t*>(base) + first * row_bytes : nullptr, scale_a + (size_t)first * sa_stride,
+                           sa_stride, scale_b, sb_stride, out_scale, m - first, n, k, b_stride, d_dtype, epilogue, nullptr, stream,
+                           packed, use_static);
+    }
     hfrk_gemm_plan p;
     if (user_plan) {
         p = *user_plan;
@@ -1090,7 +1112,7 @@ int hfrk_skinny_gemm_validate(int m, int n, int k, int b_stride, int split_k, in
     if (a_lanes > 4 || b_lanes > 6 || qsize < 1 || qsize > 6 || (ops != 4 && ops != 8)) return HFRK_INVALID_CONFIG;
     // limits of this implementation
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
-    if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (k % 16 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;  // (never after the check above: the reference's tiles are 64+ wide)
     if (b_stride % 16 != 0) return HFRK_BAD_ALIGNMENT;
     return HFRK_SUCCESS;
 }

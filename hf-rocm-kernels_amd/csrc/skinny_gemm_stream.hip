@@ -40,8 +40,14 @@ namespace hfrk {
 // 16-bit projections -- the SwiGLU kernel of csrc/op_src/swiglu/swiglu_vectorized.cu:27-97 as a GEMM epilogue.
 // PACKED: the weight is in the pre-packed layout (pack_weight.hip): chunk (tile, kc) is 4 KB at
 // (tile * KC + kc) * 4096, already in MFMA operand order, so a chunk is one contiguous read and needs no LDS pass.
-template <int MA, int RT, bool SWIGLU, bool PACKED>
+// RAGGED_K: row-major weights whose k is a multiple of 16 but not of 256: the last chunk of a row is cut short by whole
+// 16-byte pieces, and the lanes whose piece lies beyond k read zeros in both operands (the reference accepts such k
+// with its narrow tiles, csrc/op_src/skinny_gemm/skinny_gemm_caller.cu:33-48).  A variant of its own, so that the
+// common case keeps its instruction count before the first request.
+enum { kLayoutRowMajor = 0, kLayoutPacked = 1, kLayoutRaggedK = 2 };
+template <int MA, int RT, bool SWIGLU, int LAYOUT>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const GemmArgs a) {
+    constexpr bool PACKED = LAYOUT == kLayoutPacked, RAGGED_K = LAYOUT == kLayoutRaggedK;
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kCoherent = 17;  // sc0 | sc1
     constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles
@@ -80,15 +86,20 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)li * 16u;
     const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
+    // RAGGED_K: in a row's last chunk the lanes whose piece lies beyond k start from an out-of-range offset
+    const bool beyond_k = RAGGED_K && (KC - 1) * 256 + li * 16 >= a.k;
+    const uint32_t w_tail_off = beyond_k ? kOutOfRange : w_lane_off, a_tail_off = beyond_k ? kOutOfRange : a_lane_off;
     v4i wq[4 * RT], aq[MA];
     int itile = tile, ikc = kc;  // chunk being requested
     auto issue_chunk = [&]() __attribute__((always_inline)) {
         const uint32_t abase = (uint32_t)ikc * 256u;
         // row group t: weight rows [16*RT*t, 16*RT*(t+1)), or with SWIGLU rows [16t, 16t+16) and n/2 + the same
         const uint32_t wbase = (uint32_t)itile * (SWIGLU ? 16u : 16u * RT) * (uint32_t)a.b_stride + (uint32_t)ikc * 256u;
+        const bool last = RAGGED_K && ikc == KC - 1;  // uniform
+        const uint32_t a_off = last ? a_tail_off : a_lane_off, w_off = last ? w_tail_off : w_lane_off;
 #pragma unroll
         for (int t = 0; t < MA; ++t)
-            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_off + abase + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
         if constexpr (PACKED) {
             // 16-row tile of row group t: RT*t + rt, or with SWIGLU t (gate) and n/32 + t (up); a tile past the last
             // one (odd tile count, RT = 2) is out of the buffer's range and reads as zero
@@ -100,7 +111,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
         } else {
 #pragma unroll
             for (int t = 0; t < 4 * RT; ++t)
-                wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_lane_off + wbase + (uint32_t)(SWIGLU ? (t / 4) * (a.n >> 1) + 4 * (t % 4) : 4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
+                wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(w_off + wbase + (uint32_t)(SWIGLU ? (t / 4) * (a.n >> 1) + 4 * (t % 4) : 4 * t) * (uint32_t)a.b_stride), 0, 2 /* nt */);
         }
     };
     if (count > 0) issue_chunk();
@@ -411,9 +422,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_stream_kernel(const 
     }
 }
 
-template <int MA, int RT, bool SWIGLU, bool PACKED>
+template <int MA, int RT, bool SWIGLU, int LAYOUT>
 static int launch_stream_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_stream_kernel<MA, RT, SWIGLU, PACKED>;
+    auto kern = skinny_gemm_stream_kernel<MA, RT, SWIGLU, LAYOUT>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -428,8 +439,9 @@ static int launch_stream_packing(const GemmArgs& args, int lds_bytes, hipStream_
 
 template <int MA, int RT, bool SWIGLU>
 static int launch_stream_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    return args.packed ? launch_stream_packing<MA, RT, SWIGLU, true>(args, lds_bytes, stream)
-                       : launch_stream_packing<MA, RT, SWIGLU, false>(args, lds_bytes, stream);
+    if (args.packed) return launch_stream_packing<MA, RT, SWIGLU, kLayoutPacked>(args, lds_bytes, stream);
+    if (args.k % 256 != 0) return launch_stream_packing<MA, RT, SWIGLU, kLayoutRaggedK>(args, lds_bytes, stream);
+    return launch_stream_packing<MA, RT, SWIGLU, kLayoutRowMajor>(args, lds_bytes, stream);
 }
 
 int launch_stream_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream) {

@@ -106,8 +106,17 @@ class Fp8Linear(torch.nn.Module):
         self.packed = self.weight_data.dim() == 1
         self._operand = PackedWeight(self.weight_data, self.out_features, self.in_features) if self.packed else self.weight_data
 
+    _QUANTISED = ("weight_data", "weight_scale", "input_scale")
+
     def _apply(self, fn, *args, **kwargs):
+        """Device moves reach every buffer; dtype casts (`.half()`, `.to(torch.bfloat16)`) reach the bias only: the fp8
+        weight and the float32 scales are what the GEMM takes and keep their dtypes."""
+        before = {name: getattr(self, name) for name in self._QUANTISED}
         module = super()._apply(fn, *args, **kwargs)
+        for name, old in before.items():
+            new = getattr(self, name)
+            if old is not None and new is not None and new.dtype != old.dtype:
+                self._buffers[name] = old.to(new.device)
         self._refresh()
         return module
 
@@ -139,8 +148,8 @@ class Fp8Linear(torch.nn.Module):
 
 def convert_linear_layers(module: torch.nn.Module, per_channel: bool = True, packed: bool = False,
                           skip: Sequence[str] = ()) -> int:
-    """Replace, in place and recursively, every nn.Linear under `module` that the FP8 GEMM can take (in_features a
-    multiple of 256, 16-bit weight) by an Fp8Linear quantised from it; returns how many were replaced.
+    """Replace, in place and recursively, every nn.Linear under `module` that the FP8 path can take (in_features a
+    multiple of 16 -- of 256 for packed weights -- and at most 32768, 16-bit weight) by an Fp8Linear quantised from it; returns how many were replaced.
     skip: layers whose dotted name ends with one of these strings stay as they are (e.g. ("lm_head",)).
     The counterpart, without the serving stack, of switching a model's linear method (reference README.md:95-97)."""
     replaced = 0
@@ -150,7 +159,9 @@ def convert_linear_layers(module: torch.nn.Module, per_channel: bool = True, pac
         for name, child in list(parent.named_children()):
             full = f"{prefix}.{name}" if prefix else name
             if isinstance(child, torch.nn.Linear):
-                usable = child.in_features % 256 == 0 and child.weight.dtype in (torch.float16, torch.bfloat16)
+                # the activation quantiser reads a row of at most 32768 values in one pass
+                usable = (child.in_features % (256 if packed else 16) == 0 and child.in_features <= 32768
+                          and child.weight.dtype in (torch.float16, torch.bfloat16))
                 if usable and not any(full.endswith(suffix) for suffix in skip):
                     setattr(parent, name, Fp8Linear.from_float(child, per_channel=per_channel, packed=packed))
                     replaced += 1

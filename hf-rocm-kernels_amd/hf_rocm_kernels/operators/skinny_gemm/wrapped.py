@@ -52,6 +52,8 @@ def infer_skinny_gemm_m_params(m: int) -> Tuple[int, int]:
 def _planned_k_slabs(m: int, n: int, k: int) -> int:
     """K slabs per row panel in the library's plan for the shape: a host-only call into the C library, a constant
     of the shape to a tracer (which cannot follow a ctypes call)."""
+    if k % 256 and m > 32:  # no single plan: the library runs two launches of up to 32 rows
+        return (k + 255) // 256
     return int(_capi.plan(m, n, k).slabs)
 
 
@@ -66,6 +68,10 @@ def infer_skinny_gemm_params(skinny_a: Tensor, b: Tensor) -> Dict[str, int]:
     n = b.shape[1]
     a_lanes, op_m = infer_skinny_gemm_m_params(m)
     ops = 4 if op_m == 8 else 8
+    if k % 256 and k % 16 == 0:
+        # a row that ends inside a 256-byte chunk: name the reference's narrowest tile that divides k, (512/op_m)*ops =
+        # 128 or 64 (skinny_gemm_caller.cu:33-48), so that the launcher's validation passes where the reference's would
+        op_m, ops = (16, 4) if k % 128 == 0 else (32, 4)
     b_lanes = min(4, max(1, n // (256 * 16)))
     qsize = 3
     return {"A_producers": 3, "B_producers": min(6, qsize * b_lanes), "consumers": 3,
@@ -106,13 +112,13 @@ def skinny_gemm(
           or the PackedWeight made from that weight (utils/weight_format.py), here and in the variants below
         - scale_tensor: a fp32 one-item tensor, the product of the two quantisation scales
         - output: an optional (m, n) bfloat16/float16 tensor that is accumulated into: zero-initialised, or
-          holding a bias or residual.  Allocated as bfloat16 zeros when omitted.
+          holding a bias or residual.  Allocated as float16 zeros when omitted, like the reference's (wrapped.py:119).
     Outputs:
         the (m, n) output tensor.
     Unlike the reference, a launcher status other than 0 raises instead of leaving the output untouched.
     """
     if output is None:
-        output = torch.zeros(size=(skinny_a.size(0), b.size(1)), dtype=torch.bfloat16, device=skinny_a.device)
+        output = torch.zeros(size=(skinny_a.size(0), b.size(1)), dtype=torch.float16, device=skinny_a.device)
     skinny_gemm_checks(skinny_a, b, scale_tensor, output)
     if isinstance(b, PackedWeight) or torch.compiler.is_compiling():  # the 13-argument op takes the row-major view only
         _fused(skinny_a, b, output, output, scale_tensor.view(-1), None, None, _capi.EPILOGUE_NONE, 0)
@@ -132,7 +138,9 @@ def skinny_gemm_scaled(
     accumulate: bool = False,
 ) -> Tensor:
     """Per-token x per-output-channel variant: output[i, j] (+)= scale_a[i] * scale_b[j] * (skinny_a @ b)[i, j].
-    `scale_a` has 1 or m float32 elements, `scale_b` 1 or n.  With accumulate=False the output is overwritten."""
+    `scale_a` has 1 or m float32 elements, `scale_b` 1 or n.  With accumulate=False the output is overwritten.
+    This variant has no counterpart in the reference; an omitted output is allocated as bfloat16 (the serving dtype of the
+    Llama-3 checkpoints it is used with), unlike `skinny_gemm`, which keeps the reference's float16."""
     m, n = skinny_a.size(0), b.size(1)
     if output is None:
         output = torch.empty(size=(m, n), dtype=torch.bfloat16, device=skinny_a.device)

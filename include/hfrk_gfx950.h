@@ -28,7 +28,11 @@ enum hfrk_status {
     HFRK_SUCCESS = 0,
     HFRK_M_ABOVE_WARPTILE_M = 1,            /* never returned (the reference has the check commented out) */
     HFRK_N_NOT_EVEN = 2,
-    HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K = 3, /* k % ((512/op_m)*ops) != 0, or k % 256 != 0 */
+    HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K = 3, /* k % ((512/op_m)*ops) != 0; k % 16 != 0; k % 256 != 0 with a packed weight
+                                             * or with an explicit plan of another kernel than the wave-stream one
+                                             * (a variant of it handles a row that ends inside a 256-byte chunk by
+                                             * masking the missing 16-byte pieces; without a plan, calls of more
+                                             * than 32 rows then run as two launches) */
     HFRK_TOO_MANY_WARPS = 4,                /* A_producers + B_producers + consumers > 16 */
     HFRK_QSIZE_TOO_SMALL = 5,
     HFRK_INVALID_CONFIG = 6,                /* knob tuple outside the accepted domain */

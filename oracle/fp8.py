@@ -39,7 +39,9 @@ def decode(codes) -> np.ndarray:
 
 
 def encode_rne(x: np.ndarray) -> np.ndarray:
-    """float -> nearest e4m3fn code, ties to even mantissa, |x| > 448 saturating to +-448, NaN -> 0x7F.
+    """float -> nearest e4m3fn code, ties to even mantissa, |x| > 448 saturating to +-448, NaN -> 0x7F (the device
+    kernels clamp with a median-of-three that turns NaN into -448, code 0xFE, before converting: NaN inputs are the one
+    place where the two differ, pinned by a GPU test).
 
     Written against the value grid (search in the sorted table of the 127 non-negative finite values), not by
     bit manipulation, so that it is independent of torch's cast."""

@@ -121,6 +121,51 @@ def test_every_plan_gives_the_same_answer(m, n, k):
             raise AssertionError(f"plan {p.as_dict()}: {e}")
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096 + 128), (8, 1000, 640), (16, 6144, 4096 + 64), (32, 2048, 1152),
+                                   (33, 1024, 640), (64, 4096, 4096 + 128), (5, 256, 144), (3, 128, 16), (12, 4096, 1008)])
+def test_k_that_ends_inside_a_chunk(m, n, k):
+    """k % 16 == 0 but k % 256 != 0 (the reference takes such k with its narrow tiles, skinny_gemm_caller.cu:33-48): the
+    last chunk of every row is cut short.  The weight is a view of wider rows whose bytes beyond k are NaN codes, so a
+    kernel that reads past k, in either operand, cannot pass; above 32 rows the call runs as two launches."""
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    lib = _capi.load()
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k, per_token=True, per_channel=True)
+    wide = torch.full((n, k + 112), 0x7F, dtype=torch.uint8, device="cuda")
+    wide[:, :k] = b.t().contiguous().view(torch.uint8)
+    b_view = wide.view(torch.float8_e4m3fn)[:, :k].t()
+    assert b_view.stride() == (1, k + 112)
+    for weight in (b, b_view):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        run_ex(a, weight, sa, sw, out, accumulate=False)
+        check_against_oracle(out, a, b, sa, sw)
+    base = torch.randn(m, n, generator=torch.Generator().manual_seed(1)).to(torch.float16).cuda()
+    out = base.clone()
+    run_ex(a, b_view, sa, sw, out, accumulate=True)
+    check_against_oracle(out, a, b, sa, sw, base=base)
+    # every explicit plan of the kernel that cuts a chunk short; the others and the packed format refuse
+    kc = (k + 255) // 256
+    plans = [p for p in all_plans(m, n, (k // 256) * 256 or 256) if p.wn == 0] if m <= 32 else []
+    for p in plans:
+        p.slabs = kc
+        p.grid = min(p.grid, p.panels * kc)
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        try:
+            run_ex(a, b_view, sa, sw, out, accumulate=False, plan=p)
+            check_against_oracle(out, a, b, sa, sw)
+        except (AssertionError, RuntimeError) as e:
+            raise AssertionError(f"plan {p.as_dict()}: {e}")
+    refused = _capi.GemmPlan((m + 15) // 16, 8, 1, 1, 1, (n + 127) // 128, max(1, k // 256), 8 * 4096 + 2 * 16 * ((m + 15) // 16) * 256)
+    out = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    assert lib.hfrk_skinny_gemm_ex(a.data_ptr(), b.data_ptr(), out.data_ptr(), sa.data_ptr(), 1, sw.data_ptr(), 1, m, n, k, k,
+                                   _capi.BF16, 0, ctypes.byref(refused), None) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
+    assert lib.hfrk_packed_weight_bytes(n, k) == 0
+    if k % 64 == 0:  # the reference's operator: one combined scale, accumulating into float16
+        from hf_rocm_kernels import skinny_gemm
+        scale = (sa[:1] * sw[:1]).contiguous()
+        check_against_oracle(skinny_gemm(a, b_view, scale), a, b, scale, torch.ones(1).cuda())
+
+
 # ---- the operator surface: torch.ops._HFRK_C / hf_rocm_kernels.skinny_gemm ----------------------------------------
 
 @pytest.mark.parametrize("repeat_id", "abc")
@@ -158,9 +203,9 @@ def test_accumulates_into_output_like_the_reference():
     bias = torch.randn(m, n, generator=g).to(torch.bfloat16).cuda()
     out = skinny_gemm(a, b, scale, bias.clone())
     check_against_oracle(out, a, b, scale, torch.ones(1).cuda(), base=bias)
-    # output=None allocates zeros in bfloat16
+    # output=None allocates float16 zeros, as the reference does (operators/skinny_gemm/wrapped.py:119)
     out0 = skinny_gemm(a, b, scale)
-    assert out0.dtype == torch.bfloat16
+    assert out0.dtype == torch.float16
     check_against_oracle(out0, a, b, scale, torch.ones(1).cuda())
 
 
@@ -195,10 +240,10 @@ def test_full_size_properties_llama70b_down():
         hot[i, c] = 2.0
     out = skinny_gemm(hot.to(torch.float8_e4m3fn).cuda(), w.t(), torch.tensor([0.5]).cuda())
     for i, c in enumerate(cols):
-        assert torch.equal(out[i].float(), w[:, c].float().to(torch.bfloat16).float())
+        assert torch.equal(out[i].float(), w[:, c].float())   # every e4m3 value is a float16 value
     a = torch.randn(m, k, generator=g).clamp(-4, 4).to(torch.float8_e4m3fn).cuda()
-    o1 = skinny_gemm(a, w.t(), torch.tensor([2.0 ** -12]).cuda())
-    o4 = skinny_gemm(a, w.t(), torch.tensor([2.0 ** -10]).cuda())
+    o1 = skinny_gemm(a, w.t(), torch.tensor([2.0 ** -12]).cuda(), torch.zeros_like(bias))
+    o4 = skinny_gemm(a, w.t(), torch.tensor([2.0 ** -10]).cuda(), torch.zeros_like(bias))
     assert torch.equal(o4.float(), o1.float() * 4)       # power-of-two scales commute with the rounding
 
 
@@ -211,8 +256,11 @@ def test_status_codes_and_misuse():
     one = torch.ones(1).cuda()
     knobs = dict(split_k=1, A_producers=3, B_producers=4, consumers=3, a_lanes=1, b_lanes=4, qsize=3, op_m=8, ops=4)
     assert _skinny_gemm(a, b, one, d, **knobs) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K      # k = 384
+    assert torch.equal(skinny_gemm(a, b, one, d), torch.zeros_like(d))   # the wrapper names a tile that divides 384: (512/16)*4
+    a = torch.zeros(8, 392).to(torch.float8_e4m3fn).cuda()
+    b = torch.zeros(128, 392).to(torch.float8_e4m3fn).cuda().t()
     with pytest.raises(RuntimeError, match="status 3"):
-        skinny_gemm(a, b, one, d)                                                          # the wrapper raises
+        skinny_gemm(a, b, one, d)                                                          # k % 16 != 0: the wrapper raises
     a = torch.zeros(8, 256).to(torch.float8_e4m3fn).cuda()
     b = torch.zeros(127, 256).to(torch.float8_e4m3fn).cuda().t()
     d = torch.zeros(8, 127, dtype=torch.bfloat16).cuda()
@@ -407,7 +455,7 @@ def test_benchmarking_helpers_and_the_library_gemm_agree_with_scaled_mm():
     a, b, sa, sw = generate_llama_gemm_data(8, 1024, 2048, seed=12)
     ours = skinny_gemm(a, b, (sa * sw).contiguous())
     try:
-        theirs = torch._scaled_mm(a, b, scale_a=sa.reshape(1), scale_b=sw.reshape(1), out_dtype=torch.bfloat16)
+        theirs = torch._scaled_mm(a, b, scale_a=sa.reshape(1), scale_b=sw.reshape(1), out_dtype=ours.dtype)
     except Exception as e:  # not every torch build has the fp8 hipBLASLt path
         theirs = None
         print("torch._scaled_mm unavailable:", e)

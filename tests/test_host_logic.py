@@ -40,7 +40,11 @@ def test_validation_codes_match_the_reference_launcher():
     assert _validate() == _capi.SUCCESS
     assert _validate(n=4097) == _capi.N_NOT_EVEN
     assert _validate(k=4096 + 128) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K      # (512/8)*4 = 256
-    assert _validate(k=128, op_m=16, ops=4) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K  # passes the reference's 128, not this kernel's 256
+    # k that is no multiple of 256 passes wherever the reference's tile (512/op_m)*ops divides it (skinny_gemm_caller.cu:33-48)
+    assert _validate(k=128, op_m=16, ops=4) == _capi.SUCCESS
+    assert _validate(k=4096 + 128, op_m=16, ops=4) == _capi.SUCCESS
+    assert _validate(k=4096 + 64, op_m=32, ops=4) == _capi.SUCCESS
+    assert _validate(k=4096 + 64, op_m=16, ops=4) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
     assert _validate(A=6, B=6, C=5) == _capi.TOO_MANY_WARPS
     assert _validate(A=3, B=4, C=3, q=2) == _capi.QSIZE_TOO_SMALL              # consumers > qsize
     assert _validate(B=8, bl=1, q=3, A=2, C=2) == _capi.QSIZE_TOO_SMALL        # B_producers / b_lanes > qsize
@@ -235,6 +239,21 @@ def test_plan_rejects_what_the_kernel_cannot_take():
     assert lib.hfrk_skinny_gemm_plan(0, 128, 256, ctypes.byref(p)) == _capi.BAD_SHAPE
     assert lib.hfrk_skinny_gemm_plan(8, 128, 300, ctypes.byref(p)) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
     assert lib.hfrk_skinny_gemm_plan(8, 128, 256, None) == _capi.BAD_SHAPE
+
+
+def test_plans_for_k_that_ends_inside_a_chunk():
+    """k % 16 == 0 is enough for row-major weights up to 32 rows: wave-stream plans count the cut-short last chunk
+    (slabs = ceil(k / 256)); packed weights, the other kernels and single plans above 32 rows need k % 256 == 0."""
+    p = _capi.GemmPlan()
+    lib = _capi.load()
+    assert lib.hfrk_skinny_gemm_plan(8, 4096, 4096 + 128, ctypes.byref(p)) == 0
+    assert p.wn == 0 and p.slabs == 17 and p.panels == 256
+    assert lib.hfrk_skinny_gemm_plan(32, 1000, 640, ctypes.byref(p)) == 0
+    assert p.wn == 0 and p.slabs == 3
+    assert lib.hfrk_skinny_gemm_plan(8, 256, 144, ctypes.byref(p)) == 0
+    assert p.wn == 0 and p.slabs == 1
+    assert lib.hfrk_skinny_gemm_plan(33, 1000, 640, ctypes.byref(p)) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
+    assert lib.hfrk_skinny_gemm_plan(8, 1000, 648, ctypes.byref(p)) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
 
 
 def test_op_schemas_are_the_reference_schemas():
@@ -552,3 +571,36 @@ def test_c_loader_rejects_what_is_not_a_plan_table(tmp_path):
     finally:
         plan_table.clear()
         plan_table.load_from_environment()
+
+
+def test_fp8_linear_keeps_its_quantised_buffers_through_dtype_casts():
+    """`.half()` / `.to(torch.bfloat16)` on a converted model cast the bias only; the fp8 weight and its float32 scales stay
+    what the GEMM takes, through `state_dict` round trips too.  Layers the activation quantiser cannot take are left alone."""
+    from hf_rocm_kernels.layers.fp8_linear import Fp8Linear, convert_linear_layers
+    torch.manual_seed(5)
+    model = torch.nn.Sequential(torch.nn.Linear(512, 64, bias=True), torch.nn.Linear(256, 32, bias=False),
+                                torch.nn.Linear(100, 8), torch.nn.Linear(33024, 2, bias=False)).to(torch.bfloat16)
+    assert convert_linear_layers(model) == 2
+    assert isinstance(model[0], Fp8Linear) and isinstance(model[1], Fp8Linear)
+    assert isinstance(model[2], torch.nn.Linear) and isinstance(model[3], torch.nn.Linear)  # k % 256 != 0; k > 32768
+    layer = model[0]
+    layer.register_buffer("input_scale", torch.tensor([0.02]))
+    weight_bits = layer.weight_data.view(torch.uint8).clone()
+    scale = layer.weight_scale.clone()
+    for cast in (lambda mod: mod.half(), lambda mod: mod.to(torch.bfloat16), lambda mod: mod.float(), lambda mod: mod.to("cpu")):
+        cast(model)
+        assert layer.weight_data.dtype == torch.float8_e4m3fn and layer.weight_scale.dtype == torch.float32
+        assert layer.input_scale.dtype == torch.float32
+        assert torch.equal(layer.weight_data.view(torch.uint8), weight_bits) and torch.equal(layer.weight_scale, scale)
+        assert layer.weight is layer.weight_data  # the operand follows the buffer
+    model.half()
+    assert layer.bias.dtype == torch.float16
+    state = {name: t.clone() for name, t in model.state_dict().items()}
+    assert state["0.weight_data"].dtype == torch.float8_e4m3fn
+    twin = torch.nn.Sequential(torch.nn.Linear(512, 64, bias=True), torch.nn.Linear(256, 32, bias=False),
+                               torch.nn.Linear(100, 8), torch.nn.Linear(33024, 2, bias=False)).to(torch.bfloat16)
+    convert_linear_layers(twin)
+    twin[0].register_buffer("input_scale", torch.zeros(1))
+    twin.half().load_state_dict(state)
+    assert torch.equal(twin[0].weight_data.view(torch.uint8), weight_bits) and torch.equal(twin[0].weight_scale, scale)
+    assert twin[0].weight is twin[0].weight_data

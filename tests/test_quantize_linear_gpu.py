@@ -153,8 +153,8 @@ def test_checked_gemm_operator_raises_where_the_status_operator_returns_a_code()
     one = torch.ones(1, device="cuda")
     d = torch.zeros(4, 64, device="cuda", dtype=torch.bfloat16)
     torch.ops._HFRK_C.skinny_gemm_checked(a, w.t(), False, 64, d, None, one, None, None, 0, 0)
-    bad_a = torch.zeros(4, 384, device="cuda").to(torch.float8_e4m3fn)  # k not a multiple of 256
-    bad_w = torch.zeros(64, 384, device="cuda").to(torch.float8_e4m3fn)
+    bad_a = torch.zeros(4, 392, device="cuda").to(torch.float8_e4m3fn)  # k not a multiple of 16
+    bad_w = torch.zeros(64, 392, device="cuda").to(torch.float8_e4m3fn)
     assert torch.ops._HFRK_C.skinny_gemm_fused(bad_a, bad_w.t(), d, None, one, None, None, 0, 0) == 3
     with pytest.raises(RuntimeError, match="status 3"):
         torch.ops._HFRK_C.skinny_gemm_checked(bad_a, bad_w.t(), False, 64, d, None, one, None, None, 0, 0)

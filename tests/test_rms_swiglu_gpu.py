@@ -281,6 +281,35 @@ def test_swiglu_dynamic(rows, cols, dtype):
     _check_dynamic(q, scales, q_ref, s_ref, y)
 
 
+def test_nan_inputs_quantise_like_the_reference_clamp():
+    """A NaN does not survive the device's clamp to +-448 (a median of three returns the smaller of the two bounds): it
+    is stored as -448 (0xFE), as the reference's clamp stores it, not as the 0x7F the CPU oracle's encoder writes.  The
+    dynamic quantiser's row maximum ignores NaN, so the row's scale stays finite and its other values keep their codes."""
+    from hf_rocm_kernels import swiglu, swiglu_dynamic
+    from oracle import swiglu as osw
+    g = torch.Generator().manual_seed(11)
+    gu = torch.randn(3, 64, generator=g).to(torch.bfloat16)
+    gu[1, 5] = float("nan")        # a gate value
+    gu[2, 32 + 9] = float("nan")   # an up value
+    scale = torch.tensor([0.05])
+    for force_scalar in (False, True):
+        out = swiglu(gu.cuda(), scale.cuda(), None, force_scalar=force_scalar).cpu().view(torch.uint8)
+        assert out[1, 5] == 0xFE and out[2, 9] == 0xFE
+        clean = gu.clone()
+        clean[1, 5] = clean[2, 32 + 9] = 0.0
+        ref = osw.reference_swiglu(clean, scale).view(torch.uint8)
+        mask = torch.ones(3, 32, dtype=torch.bool)
+        mask[1, 5] = mask[2, 9] = False
+        assert (out[mask].int() - ref[mask].int()).abs().max() <= 1
+    q, scales = swiglu_dynamic(gu.cuda())
+    assert torch.isfinite(scales).all()
+    q = q.cpu().view(torch.uint8)
+    assert q[1, 5] == 0xFE and q[2, 9] == 0xFE
+    q_ref, s_ref, _ = osw.precise_swiglu_dynamic(clean)
+    assert torch.allclose(scales.cpu().reshape(-1), s_ref.reshape(-1).float(), rtol=1e-5)
+    assert (q[mask].int() - q_ref.view(torch.uint8)[mask].int()).abs().max() <= 1
+
+
 def test_dynamic_scales_feed_the_gemm():
     """rms_dynamic -> per-token GEMM: the device's own fp8 rows and scales through the GEMM oracle."""
     from hf_rocm_kernels import residual_rms_dynamic, skinny_gemm_scaled
