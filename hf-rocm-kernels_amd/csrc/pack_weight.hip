@@ -140,6 +140,12 @@ static int launch_pack(const void* src, void* dst, int n, int k, int row_stride,
     return HFRK_SUCCESS;
 }
 
+// the per-output-channel scales behind the packed bytes: n values, then zeros up to the padded row count
+__global__ void pack_scales_kernel(const float* __restrict__ src, float* __restrict__ dst, int n, int n_padded) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_padded) dst[i] = i < n ? src[i] : 0.0f;
+}
+
 }  // namespace hfrk
 
 extern "C" {
@@ -147,6 +153,30 @@ extern "C" {
 size_t hfrk_packed_weight_bytes(int n, int k) {
     if (n < 1 || k < 1 || k % 256 != 0) return 0;
     return (size_t)((n + 15) / 16) * 16 * (size_t)k;
+}
+
+size_t hfrk_packed_weight_bytes_scaled(int n, int k) {
+    const size_t bytes = hfrk_packed_weight_bytes(n, k);
+    return bytes ? bytes + (size_t)((n + 15) / 16) * 16 * sizeof(float) : 0;
+}
+
+const float* hfrk_packed_weight_scales(const void* packed, int n, int k) {
+    const size_t bytes = hfrk_packed_weight_bytes(n, k);
+    return (bytes && packed) ? reinterpret_cast<const float*>(static_cast<const uint8_t*>(packed) + bytes) : nullptr;
+}
+
+int hfrk_pack_weight_scaled(const void* src, int src_stride, int src_format, const float* scales, void* dst, int n, int k,
+                            void* stream) {
+    if (!scales) return HFRK_BAD_SHAPE;
+    if (reinterpret_cast<uintptr_t>(scales) & 3) return HFRK_BAD_ALIGNMENT;
+    const int rc = hfrk_pack_weight(src, src_stride, src_format, dst, n, k, stream);
+    if (rc != HFRK_SUCCESS) return rc;
+    const int n_padded = (n + 15) / 16 * 16;
+    float* tail = const_cast<float*>(hfrk_packed_weight_scales(dst, n, k));
+    hipLaunchKernelGGL(hfrk::pack_scales_kernel, dim3((n_padded + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       scales, tail, n, n_padded);
+    HFRK_HIP_TRY(hipGetLastError());
+    return HFRK_SUCCESS;
 }
 
 int hfrk_pack_weight(const void* src, int src_stride, int src_format, void* dst, int n, int k, void* stream) {

@@ -1181,6 +1181,11 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
 int hfrk_skinny_gemm_packed(const void* A, const void* B_packed, void* D, const void* base, const float* scale_a,
                             int sa_stride, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
                             int k, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
+    if (sb_stride == HFRK_SCALES_IN_PACKED_BUFFER) {  // the per-channel scales hfrk_pack_weight_scaled stored behind the bytes
+        scale_b = hfrk_packed_weight_scales(B_packed, n, k);
+        if (!scale_b) return k % 256 != 0 ? HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K : HFRK_BAD_SHAPE;
+        sb_stride = 1;
+    }
     return hfrk::gemm_launch(A, B_packed, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, m, n, k, k, d_dtype,
                              epilogue, plan, static_cast<hipStream_t>(stream), true);
 }

@@ -272,10 +272,13 @@ int64_t gemm_fused_common(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, 
     TORCH_CHECK(A.dim() == 2 && A.is_contiguous(), "A must be a contiguous [m, k] tensor");
     check_fp8(A, "A");
     check_fp8(B, "B");
+    bool scales_in_buffer = false;  // a buffer of pack_weight_scaled: its per-channel scales apply when scale_b is None
     if (packed) {
         TORCH_CHECK(n >= 1 && n < (int64_t(1) << 30) && A.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
-        TORCH_CHECK(B.is_contiguous() && (size_t)B.numel() == hfrk_packed_weight_bytes((int)n, (int)A.size(1)) && B.numel() > 0,
-                    "B must be the packed buffer of a [n, k] weight (pack_weight) with k = A.size(1)");
+        const size_t plain = hfrk_packed_weight_bytes((int)n, (int)A.size(1)), scaled = hfrk_packed_weight_bytes_scaled((int)n, (int)A.size(1));
+        TORCH_CHECK(B.is_contiguous() && B.numel() > 0 && ((size_t)B.numel() == plain || (size_t)B.numel() == scaled),
+                    "B must be the packed buffer of a [n, k] weight (pack_weight, pack_weight_scaled) with k = A.size(1)");
+        scales_in_buffer = (size_t)B.numel() == scaled;
     } else {
         TORCH_CHECK(B.dim() == 2 && B.size(0) == A.size(1) && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
     }
@@ -293,6 +296,8 @@ int64_t gemm_fused_common(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, 
         check_same_device(A, *scale_b, "scale_b");
         scale_b_ptr = scale_b->data_ptr<float>();
         sb_stride = scale_b->numel() == 1 ? 0 : 1;
+    } else if (scales_in_buffer) {
+        sb_stride = HFRK_SCALES_IN_PACKED_BUFFER;
     }
     int d_dtype;
     const void* base_ptr = nullptr;
@@ -369,12 +374,28 @@ void pack_weight(at::Tensor& src, at::Tensor& dst, int64_t src_format) {
     raise_on(hfrk_pack_weight(src.data_ptr(), (int)src.stride(0), (int)src_format, dst.data_ptr(), n, k, current_stream(src)), "pack_weight");
 }
 
+// The same with the weight's per-output-channel scales stored behind the packed bytes (one allocation per layer).
+void pack_weight_scaled(at::Tensor& src, at::Tensor& scales, at::Tensor& dst, int64_t src_format) {
+    TORCH_CHECK(src.dim() == 2 && src.stride(1) == 1 && is_byte_tensor(src), "src must be a [n, k] one-byte tensor with unit stride along k");
+    TORCH_CHECK(src.size(0) < (int64_t(1) << 30) && src.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
+    const int n = (int)src.size(0), k = (int)src.size(1);
+    TORCH_CHECK(scales.scalar_type() == at::kFloat && scales.is_contiguous() && scales.numel() == n, "scales must be n contiguous float32 values");
+    TORCH_CHECK(is_byte_tensor(dst) && dst.is_contiguous() && (size_t)dst.numel() == hfrk_packed_weight_bytes_scaled(n, k) && dst.numel() > 0,
+                "dst must be a contiguous one-byte tensor of hfrk_packed_weight_bytes_scaled(n, k) elements (k % 256 == 0)");
+    check_same_device(src, dst, "dst");
+    check_same_device(src, scales, "scales");
+    DeviceScope scope(src);
+    raise_on(hfrk_pack_weight_scaled(src.data_ptr(), (int)src.stride(0), (int)src_format, scales.data_ptr<float>(), dst.data_ptr(), n, k,
+                                     current_stream(src)), "pack_weight_scaled");
+}
+
 void unpack_weight(at::Tensor& src, at::Tensor& dst) {
     TORCH_CHECK(dst.dim() == 2 && dst.stride(1) == 1 && is_byte_tensor(dst), "dst must be a [n, k] one-byte tensor with unit stride along k");
     TORCH_CHECK(dst.size(0) < (int64_t(1) << 30) && dst.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
     const int n = (int)dst.size(0), k = (int)dst.size(1);
-    TORCH_CHECK(is_byte_tensor(src) && src.is_contiguous() && (size_t)src.numel() == hfrk_packed_weight_bytes(n, k) && src.numel() > 0,
-                "src must be a contiguous one-byte tensor of hfrk_packed_weight_bytes(n, k) elements (k % 256 == 0)");
+    TORCH_CHECK(is_byte_tensor(src) && src.is_contiguous() && src.numel() > 0 &&
+                    ((size_t)src.numel() == hfrk_packed_weight_bytes(n, k) || (size_t)src.numel() == hfrk_packed_weight_bytes_scaled(n, k)),
+                "src must be a contiguous one-byte tensor of hfrk_packed_weight_bytes(n, k) elements (k % 256 == 0), or that plus its scales");
     check_same_device(src, dst, "dst");
     DeviceScope scope(src);
     raise_on(hfrk_unpack_weight(src.data_ptr(), dst.data_ptr(), (int)dst.stride(0), n, k, current_stream(src)), "unpack_weight");
@@ -430,6 +451,8 @@ TORCH_LIBRARY(_HFRK_C, ops) {
 
     ops.def("pack_weight(Tensor src, Tensor! dst, int src_format) -> ()");
     ops.impl("pack_weight", c10::kCUDA, &pack_weight);
+    ops.def("pack_weight_scaled(Tensor src, Tensor scales, Tensor! dst, int src_format) -> ()");
+    ops.impl("pack_weight_scaled", c10::kCUDA, &pack_weight_scaled);
     ops.def("unpack_weight(Tensor src, Tensor! dst) -> ()");
     ops.impl("unpack_weight", c10::kCUDA, &unpack_weight);
     ops.def("reencode_fnuz(Tensor src, Tensor! dst) -> ()");

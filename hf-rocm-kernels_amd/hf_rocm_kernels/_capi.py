@@ -40,6 +40,7 @@ WEIGHT_E4M3FN = 0
 WEIGHT_E4M3FNUZ = 1
 
 GEMM_MAX_M = 64
+SCALES_IN_PACKED_BUFFER = -1  # sb_stride of hfrk_skinny_gemm_packed: use the scales hfrk_pack_weight_scaled stored
 
 
 class GemmPlan(ctypes.Structure):
@@ -75,6 +76,9 @@ SIGNATURES = {
     "hfrk_pack_weight": (_i, [_p, _i, _i, _p, _i, _i, _p]),
     "hfrk_unpack_weight": (_i, [_p, _p, _i, _i, _i, _p]),
     "hfrk_reencode_fnuz": (_i, [_p, _p, ctypes.c_size_t, _p]),
+    "hfrk_packed_weight_bytes_scaled": (ctypes.c_size_t, [_i, _i]),
+    "hfrk_pack_weight_scaled": (_i, [_p, _i, _i, _p, _p, _i, _i, _p]),
+    "hfrk_packed_weight_scales": (_p, [_p, _i, _i]),
     "hfrk_skinny_gemm_packed": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_residual_rms": (_i, [_p, _p, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
     "hfrk_swiglu": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),

@@ -31,7 +31,7 @@ def _weight_view(weight: Weight) -> Weight:
 def apply_fp8_linear(
     input: Tensor,
     weight: Weight,
-    weight_scale: Tensor,
+    weight_scale: Optional[Tensor],
     input_scale: Optional[Tensor] = None,
     bias: Optional[Tensor] = None,
     residual: Optional[Tensor] = None,
@@ -42,7 +42,8 @@ def apply_fp8_linear(
     - input: (..., k) float16/bfloat16 activations, quantised here -- with `input_scale` (one float32: static) or,
       when it is None, dynamically per token -- or a float8_e4m3fn tensor already quantised, `input_scale` then being
       its scale(s): one float32 or one per token
-    - weight: (n, k) float8_e4m3fn row-major, or its PackedWeight; weight_scale: one float32 or one per output channel
+    - weight: (n, k) float8_e4m3fn row-major, or its PackedWeight; weight_scale: one float32 or one per output channel,
+      or None for a PackedWeight that carries its scales
     - bias: (n,) in the output dtype; residual: (..., n) in the output dtype, added in the GEMM's epilogue (fp32 sum
       with the product, one rounding).  Given both, the bias is added to the residual first (one 16-bit add).
     - out_dtype: float16/bfloat16; defaults to the input's (bfloat16 for an fp8 input)
@@ -60,7 +61,7 @@ def apply_fp8_linear(
         sa = sa.reshape(-1)
     w = _weight_view(weight)
     n = w.size(1)
-    sb = weight_scale.reshape(-1)
+    sb = None if weight_scale is None else weight_scale.reshape(-1)
     m = q.size(0)
     base = None
     if residual is not None:
@@ -87,12 +88,14 @@ class Fp8Linear(torch.nn.Module):
 
     The tensors are registered buffers (`weight_data`, `weight_scale`, `bias`, `input_scale`), so the layer moves with
     `.to()` and round-trips through `state_dict()` / `load_state_dict()`; `weight_data` is the (n, k) fp8 weight or,
-    packed, the flat buffer of its PackedWeight (its rank tells which)."""
+    packed, the flat buffer of its PackedWeight (its rank tells which).  A packed weight with per-channel scales keeps
+    them in that same buffer (one allocation per layer) and `weight_scale` is None."""
 
-    def __init__(self, weight: Weight, weight_scale: Tensor, bias: Optional[Tensor] = None,
+    def __init__(self, weight: Weight, weight_scale: Optional[Tensor], bias: Optional[Tensor] = None,
                  input_scale: Optional[Tensor] = None):
         super().__init__()
         self.packed = isinstance(weight, PackedWeight)
+        assert weight_scale is not None or (self.packed and weight.scales is not None), "a weight without scales of its own needs weight_scale"
         self.out_features, self.in_features = (weight.n, weight.k) if self.packed else tuple(weight.shape)
         self.register_buffer("weight_data", weight.data if self.packed else weight)
         self.register_buffer("weight_scale", weight_scale)
@@ -132,9 +135,11 @@ class Fp8Linear(torch.nn.Module):
         w = linear.weight.detach()
         scale = amax_scale(w, dim=1 if per_channel else None)
         q, _ = fp8_quantize(w, scale)
-        weight = pack_weight(q) if packed else q
+        scale = scale.reshape(-1).contiguous()
         bias = None if linear.bias is None else linear.bias.detach().clone()
-        return cls(weight, scale.reshape(-1).contiguous(), bias, input_scale)
+        if packed and per_channel:
+            return cls(pack_weight(q, scale), None, bias, input_scale)
+        return cls(pack_weight(q) if packed else q, scale, bias, input_scale)
 
     def forward(self, input: Tensor, input_scale: Optional[Tensor] = None, residual: Optional[Tensor] = None) -> Tensor:
         """`input` 16-bit (quantised here) or fp8 with `input_scale`; `residual` is added in the GEMM's epilogue."""

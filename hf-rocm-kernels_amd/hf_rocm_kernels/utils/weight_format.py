@@ -5,6 +5,7 @@ No counterpart in the reference, whose kernel reads the row-major weight through
 e4m3fnuz with a doubled scale (hf_rocm_kernels/utils/fp8.py:17-29).  Here:
 
   pack_weight(weight)        [n, k] float8_e4m3fn (or float8_e4m3fnuz, re-encoded on the way) -> PackedWeight
+  pack_weight(weight, scales) the same with the n per-output-channel scales behind the bytes: one allocation per layer
   unpack_weight(packed)      back to a row-major [n, k] float8_e4m3fn tensor
   reencode_fnuz(tensor)      float8_e4m3fnuz -> float8_e4m3fn with the same values (scales unchanged)
   fnuz_bits_as_ocp(q, scale) zero-copy alternative for tensors written by the reference's fp8_quantize
@@ -12,7 +13,7 @@ e4m3fnuz with a doubled scale (hf_rocm_kernels/utils/fp8.py:17-29).  Here:
 A PackedWeight goes wherever the GEMM wrappers take `b`: skinny_gemm, skinny_gemm_scaled, skinny_gemm_add,
 skinny_gemm_swiglu and llama_mlp_combined_ops.  Results are bit-identical to the row-major weight's.
 """
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 from torch import Tensor
@@ -29,12 +30,16 @@ class PackedWeight:
     """A [n, k] fp8 weight in the packed load format (16-row x 256-byte chunks in matrix-core operand order).
 
     Quacks like the `[k, n]` column-major view the GEMM wrappers expect (`shape`, `size`, `stride`, `dtype`,
-    `device`), so their argument checks apply unchanged; `data` is the flat float8_e4m3fn buffer."""
+    `device`), so their argument checks apply unchanged; `data` is the flat float8_e4m3fn buffer.  A buffer made
+    with scales is longer by 4 bytes per padded row; `scales` is then the float32 view of its n per-channel scales,
+    which the GEMM wrappers use when they are given no `scale_b`."""
 
     def __init__(self, data: Tensor, n: int, k: int):
         assert data.dim() == 1 and data.is_contiguous() and data.dtype == FP8_DTYPE, "data must be a flat float8_e4m3fn tensor"
-        assert data.numel() == packed_weight_bytes(n, k), f"{data.numel()} bytes do not hold a packed [{n}, {k}] weight"
+        plain = packed_weight_bytes(n, k)
+        assert data.numel() in (plain, packed_weight_bytes(n, k, scaled=True)), f"{data.numel()} bytes do not hold a packed [{n}, {k}] weight"
         self.data, self.n, self.k = data, int(n), int(k)
+        self.scales: Optional[Tensor] = None if data.numel() == plain else data[plain:].view(torch.float32)[:n]
 
     @property
     def shape(self) -> Tuple[int, int]:
@@ -62,25 +67,31 @@ class PackedWeight:
         return f"PackedWeight(n={self.n}, k={self.k}, device={self.device})"
 
 
-def packed_weight_bytes(n: int, k: int) -> int:
-    """Size of the packed buffer of a [n, k] weight: rows padded to a multiple of 16 (k must be a multiple of 256)."""
-    size = _capi.load().hfrk_packed_weight_bytes(int(n), int(k))
+def packed_weight_bytes(n: int, k: int, scaled: bool = False) -> int:
+    """Size of the packed buffer of a [n, k] weight: rows padded to a multiple of 16 (k must be a multiple of 256);
+    scaled: with one float32 scale per padded row behind the bytes."""
+    lib = _capi.load()
+    size = lib.hfrk_packed_weight_bytes_scaled(int(n), int(k)) if scaled else lib.hfrk_packed_weight_bytes(int(n), int(k))
     if size == 0:
         raise ValueError(f"a [{n}, {k}] weight cannot be packed: sizes must be positive and k a multiple of 256")
     return size
 
 
-def pack_weight(weight: Tensor) -> PackedWeight:
+def pack_weight(weight: Tensor, scales: Optional[Tensor] = None) -> PackedWeight:
     """Pack a row-major [n, k] weight (an nn.Linear weight; rows may be strided, k contiguous).
     float8_e4m3fnuz input is re-encoded to float8_e4m3fn values on the way (see reencode_fnuz); uint8 is taken as
-    float8_e4m3fn bits."""
+    float8_e4m3fn bits.  scales: the weight's n float32 per-output-channel scales, stored behind the packed bytes."""
     assert weight.dim() == 2 and weight.stride(1) == 1, f"Expected a [n, k] weight with unit stride along k but got {weight.stride() = }"
     assert weight.dtype in _BYTE_DTYPES, f"Expected a one-byte dtype but got {weight.dtype = }"
     assert weight.device.type == "cuda", f"Expected a device tensor but got {weight.device = }"
     n, k = weight.shape
-    data = torch.empty(packed_weight_bytes(n, k), dtype=FP8_DTYPE, device=weight.device)
+    data = torch.empty(packed_weight_bytes(n, k, scaled=scales is not None), dtype=FP8_DTYPE, device=weight.device)
     src_format = _capi.WEIGHT_E4M3FNUZ if weight.dtype == torch.float8_e4m3fnuz else _capi.WEIGHT_E4M3FN
-    torch.ops._HFRK_C.pack_weight(weight, data, src_format)
+    if scales is None:
+        torch.ops._HFRK_C.pack_weight(weight, data, src_format)
+    else:
+        assert scales.dtype == torch.float32 and scales.numel() == n, f"Expected {n} float32 scales but got {scales.shape = }, {scales.dtype = }"
+        torch.ops._HFRK_C.pack_weight_scaled(weight, scales.reshape(-1).contiguous(), data, src_format)
     return PackedWeight(data, n, k)
 
 

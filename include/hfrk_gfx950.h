@@ -214,14 +214,26 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
  * hfrk_unpack_weight: the inverse (padding rows dropped); pack then unpack returns the source bytes.
  * hfrk_reencode_fnuz: count bytes of e4m3fnuz -> e4m3fn with the same values (dst may be src).  Exact for every
  *   code except magnitudes below 2^-6, which land on fn's subnormal grid of 2^-9 (round to nearest even); the
- *   fnuz NaN 0x80 becomes the fn NaN 0x7f.  Scales stay as they are. */
+ *   fnuz NaN 0x80 becomes the fn NaN 0x7f.  Scales stay as they are.
+ * A layer's per-output-channel scales can live in the same allocation, behind the packed bytes:
+ * hfrk_packed_weight_bytes_scaled: hfrk_packed_weight_bytes + 4 bytes per padded row (16 * ceil(n/16) float32).
+ * hfrk_pack_weight_scaled: hfrk_pack_weight, then scales[0..n) copied behind the bytes (zeros for the padding rows).
+ * hfrk_packed_weight_scales: where they are, packed + hfrk_packed_weight_bytes(n, k) (NULL if that is 0).  Host only.
+ *   The unscaled functions work on the front part of such a buffer unchanged. */
 size_t hfrk_packed_weight_bytes(int n, int k);
 int hfrk_pack_weight(const void* src, int src_stride, int src_format, void* dst, int n, int k, void* stream);
 int hfrk_unpack_weight(const void* src, void* dst, int dst_stride, int n, int k, void* stream);
 int hfrk_reencode_fnuz(const void* src, void* dst, size_t count, void* stream);
+size_t hfrk_packed_weight_bytes_scaled(int n, int k);
+int hfrk_pack_weight_scaled(const void* src, int src_stride, int src_format, const float* scales, void* dst, int n, int k,
+                            void* stream);
+const float* hfrk_packed_weight_scales(const void* packed, int n, int k);
 
 /* hfrk_skinny_gemm_fused on a packed weight: same results bit for bit (same operands, same order of sums), B is
- * the buffer hfrk_pack_weight wrote for this n and k.  With the SwiGLU epilogue n % 32 == 0 as before. */
+ * the buffer hfrk_pack_weight wrote for this n and k.  With the SwiGLU epilogue n % 32 == 0 as before.
+ * sb_stride HFRK_SCALES_IN_PACKED_BUFFER: B is a buffer of hfrk_pack_weight_scaled and its per-channel scales are
+ * used; scale_b is ignored. */
+#define HFRK_SCALES_IN_PACKED_BUFFER (-1)
 int hfrk_skinny_gemm_packed(const void* A, const void* B_packed, void* D, const void* base, const float* scale_a,
                             int sa_stride, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
                             int k, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);

@@ -308,3 +308,79 @@ def test_packed_gemm_replays_in_a_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, want)
+
+
+# ---- per-channel scales carried in the packed buffer ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("m,n,k", [(8, 4096, 4096), (3, 1000, 1024), (33, 50, 256), (16, 2080, 2048)])
+def test_scales_stored_behind_the_packed_bytes(m, n, k):
+    """hfrk_pack_weight_scaled: the packed bytes, then the n per-channel scales (zeros up to the padded row count), in one
+    buffer.  The GEMM told to use them (sb_stride = HFRK_SCALES_IN_PACKED_BUFFER through the C ABI, scale_b = None in
+    Python) gives the bits of the GEMM that is handed the scales separately, on the packed and on the row-major weight."""
+    from hf_rocm_kernels import skinny_gemm_add, skinny_gemm_scaled
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    from hf_rocm_kernels.utils.weight_format import PackedWeight, pack_weight, packed_weight_bytes, unpack_weight
+    lib, _capi = _lib()
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=n + k, per_token=True, per_channel=True)
+    w = b.t()
+    plain, scaled = packed_weight_bytes(n, k), packed_weight_bytes(n, k, scaled=True)
+    n_pad = (n + 15) // 16 * 16
+    assert scaled == plain + 4 * n_pad == lib.hfrk_packed_weight_bytes_scaled(n, k)
+    # through the C ABI, into a buffer of a known fill
+    buf = torch.full((scaled,), 0xAB, dtype=torch.uint8, device="cuda")
+    _capi.check(lib.hfrk_pack_weight_scaled(w.data_ptr(), w.stride(0), 0, sw.data_ptr(), buf.data_ptr(), n, k, None), "hfrk_pack_weight_scaled")
+    torch.cuda.synchronize()
+    assert torch.equal(buf[:plain], _pack(w.contiguous().view(torch.uint8)))
+    tail = buf[plain:].view(torch.float32)
+    assert torch.equal(tail[:n], sw) and (tail[n:] == 0).all() and tail.numel() == n_pad
+    assert lib.hfrk_packed_weight_scales(buf.data_ptr(), n, k) == buf.data_ptr() + plain
+    assert lib.hfrk_packed_weight_scales(buf.data_ptr(), n, k + 16) is None and lib.hfrk_packed_weight_bytes_scaled(n, k + 16) == 0
+    assert lib.hfrk_pack_weight_scaled(w.data_ptr(), w.stride(0), 0, None, buf.data_ptr(), n, k, None) == _capi.BAD_SHAPE
+    want = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    _run_fused(a, b, want, None, sa, sw, None, _capi.EPILOGUE_NONE, None, None)
+    check_against_oracle(want, a, b, sa, sw)
+    got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    status = lib.hfrk_skinny_gemm_packed(a.data_ptr(), buf.data_ptr(), got.data_ptr(), None, sa.data_ptr(), 1, None,
+                                         _capi.SCALES_IN_PACKED_BUFFER, None, m, n, k, _capi.BF16, _capi.EPILOGUE_NONE, None, None)
+    _capi.check(status, "hfrk_skinny_gemm_packed")
+    torch.cuda.synchronize()
+    with one_plan_for_both_layouts((m, n, k)):
+        _run_fused(a, b, want, None, sa, sw, None, _capi.EPILOGUE_NONE, None, None)
+        status = lib.hfrk_skinny_gemm_packed(a.data_ptr(), buf.data_ptr(), got.data_ptr(), None, sa.data_ptr(), 1, None,
+                                             _capi.SCALES_IN_PACKED_BUFFER, None, m, n, k, _capi.BF16, _capi.EPILOGUE_NONE, None, None)
+        _capi.check(status, "hfrk_skinny_gemm_packed")
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+    # the Python surface
+    pw = pack_weight(w, sw)
+    assert isinstance(pw, PackedWeight) and pw.data.numel() == scaled and torch.equal(pw.scales, sw)
+    assert torch.equal(pw.data.view(torch.uint8), buf)
+    assert torch.equal(unpack_weight(pw).view(torch.uint8), w.contiguous().view(torch.uint8))
+    check_against_oracle(skinny_gemm_scaled(a, pw, sa, None), a, b, sa, sw)
+    assert torch.equal(skinny_gemm_scaled(a, pw, sa, None), skinny_gemm_scaled(a, pack_weight(w), sa, sw))
+    base = torch.randn(m, n, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
+    assert torch.equal(skinny_gemm_add(a, pw, sa, None, base), skinny_gemm_add(a, pack_weight(w), sa, sw, base))
+    # scales handed over explicitly win over the stored ones
+    other = (sw * 2).contiguous()
+    assert torch.equal(skinny_gemm_scaled(a, pw, sa, other), skinny_gemm_scaled(a, pack_weight(w), sa, other))
+    with pytest.raises(AssertionError):
+        skinny_gemm_scaled(a, pack_weight(w), sa, None)
+
+
+def test_fp8_linear_keeps_packed_weight_and_scales_in_one_buffer():
+    from hf_rocm_kernels.layers import Fp8Linear
+    torch.manual_seed(4)
+    lin = torch.nn.Linear(1024, 520, bias=True).to(torch.bfloat16).cuda()
+    layer = Fp8Linear.from_float(lin, per_channel=True, packed=True)
+    assert layer.weight_scale is None and layer.weight.scales is not None and layer.weight.scales.numel() == 520
+    assert set(layer.state_dict()) == {"weight_data", "bias"}
+    apart = Fp8Linear.from_float(lin, per_channel=True, packed=False)
+    assert torch.equal(layer.weight.scales, apart.weight_scale)
+    x = torch.randn(9, 1024, device="cuda").to(torch.bfloat16)
+    want = lin(x).float()
+    got = layer(x)
+    assert (got.float() - want).norm() / want.norm() < 0.06
+    twin = Fp8Linear.from_float(torch.nn.Linear(1024, 520, bias=True).to(torch.bfloat16).cuda(), per_channel=True, packed=True)
+    twin.load_state_dict(layer.state_dict())
+    assert torch.equal(twin(x), got)
+    assert torch.equal(layer.half().to("cuda")(x), got)  # the cast reaches the bias only (x stays bfloat16: so does the output)
