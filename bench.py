@@ -67,8 +67,8 @@ WORKLOADS = {
         "text": "llama3-8b decode linears: M in {1,2,4,8,16} x qkv(6144,4096) o_proj(4096,4096) gate_up(28672,4096) "
                 "down(4096,14336); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-8B decode shapes, M=1..16 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel (16 of the 20 launches of a step); with the shipped plan table "
-                  "hfrk::skinny_gemm_kernel<1,8,1,2,1> on gate_up at M=8,16 and hfrk::skinny_gemm_ksplit_kernel<1,512> on qkv at M=16",
+        "kernel": "hfrk::skinny_gemm_rows_kernel<act_loads, row_tiles, swiglu> (all 20 launches of a step: the row-split "
+                  "wave-stream kernel, a band of weight rows and all of K per workgroup)",
     },
     "llama3-70b": {
         "shapes": [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192), ("down", 8192, 28672)],
@@ -76,8 +76,8 @@ WORKLOADS = {
         "text": "llama3-70b decode linears: M in {1,4,8,16,32} x qkv(10240,8192) o_proj(8192,8192) gate_up(57344,8192) "
                 "down(8192,28672); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-70B decode shapes, M=1..32 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel (M<=8), stream / workgroup kernel by plan table (M=16), "
-                  "hfrk::skinny_gemm_kernel / skinny_gemm_ksplit_kernel (M=32)",
+        "kernel": "hfrk::skinny_gemm_rows_kernel (M<=16; down at M=16: hfrk::skinny_gemm_kernel by plan table), "
+                  "hfrk::skinny_gemm_kernel<2,WN,WK,CH,RT> (M=32)",
     },
     "scaled-m": {
         "shapes": [("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)],
@@ -85,7 +85,7 @@ WORKLOADS = {
         "text": "M in {16,32,64} x (4096,4096) (28672,4096) (4096,14336); FP8 e4m3fn, per-token activation scales "
                 "(rows 1 and M-1 are 20x outliers) and per-output-channel weight scales, bf16 out; 9 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s, per-token x per-channel scales, M=16..64 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel / skinny_gemm_kernel (M=16), hfrk::skinny_gemm_ksplit_kernel (M=32,64 on K=4096), "
+        "kernel": "hfrk::skinny_gemm_rows_kernel (M=16), hfrk::skinny_gemm_ksplit_kernel (M=32,64 on K=4096), "
                   "hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64 on K=14336 and plan-table entries)",
     },
     "llama31-405b-tp8": {
@@ -95,7 +95,7 @@ WORKLOADS = {
                 "hf_rocm_kernels/operators/skinny_gemm/wrapped.py:45-88): M in {8,16,32} x o_proj(16384,2048) qkv(2304,16384) "
                 "gate_up(13312,16384) down(16384,6656); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 12 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over the reference's tuned shard shapes, M=8..32 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_stream_kernel / hfrk::skinny_gemm_kernel by plan table",
+        "kernel": "hfrk::skinny_gemm_rows_kernel (M<=16) / hfrk::skinny_gemm_kernel (M=32), some by plan table",
         # microseconds the reference's source comments give for its own kernel on these shapes and M buckets
         # (wrapped.py:49,60,63,66,74,77,82; measured by its authors on MI300X, 5.3 TB/s HBM3)
         "reference_us": {("o_proj", 8): 11.114, ("qkv", 8): 12.485, ("qkv", 16): 14.301, ("qkv", 32): 17.220,
@@ -569,6 +569,9 @@ def main():
     ap.add_argument("--detail", action="store_true", help="kept for older command lines: the per-case table is on by default")
     ap.add_argument("--no-cases", action="store_true", help="skip the per-case table after the timed steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--ms", type=str, default=None,
+                    help="comma-separated activation row counts replacing the workload's own (e.g. 32,64 for the MLP block above 16 rows); "
+                         "the result then describes that variant of the workload, not BASELINE's")
     ap.add_argument("--packed", action="store_true",
                     help="weights in the library's packed load format (hfrk_pack_weight) instead of row-major [N, K]")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
@@ -588,6 +591,14 @@ def main():
     if args.workload == "floor":
         print(json.dumps(run_floor_workload(torch, args)))
         return
+    if args.ms:
+        rows = [int(x) for x in args.ms.split(",")]
+        assert rows and all(1 <= r <= 64 for r in rows), "--ms takes row counts between 1 and 64"
+        MLP["ms"] = rows
+        MLP["text"] = MLP["text"].replace("M in {1,8,16}", "M in {" + ",".join(map(str, rows)) + "}")
+        if args.workload in WORKLOADS:
+            WORKLOADS[args.workload]["ms"] = rows
+            WORKLOADS[args.workload]["text"] += " [--ms " + args.ms + "]"
     is_mlp = args.workload in ("mlp", "mlp-fused")
     if is_mlp:
         fused = args.workload == "mlp-fused"
@@ -598,8 +609,10 @@ def main():
         calls, text, metric = (3 if fused else 4) * len(MLP["ms"]), MLP["text"], MLP["metric"]
         if fused:
             text = text.replace("3 blocks = 12 launches", "fused into 3 launches per block: 3 blocks = 9 launches")
-        kernel = ("residual_rms_vec_kernel + skinny_gemm_stream_kernel<MA,2,swiglu> + skinny_gemm_stream_kernel" if fused else
-                  "residual_rms_vec_kernel + skinny_gemm_stream_kernel + swiglu_vec_kernel + skinny_gemm_stream_kernel")
+        kernel = ("residual_rms_vec_kernel + skinny_gemm_rows_kernel<MA,2,swiglu> + skinny_gemm_rows_kernel" if fused else
+                  "residual_rms_vec_kernel + skinny_gemm_rows_kernel + swiglu_vec_kernel + skinny_gemm_rows_kernel")
+        if args.packed:  # the packed format is read by the wave-stream kernel
+            kernel = kernel.replace("rows_kernel", "stream_kernel")
         n_copies = MLP["cycle"]
     else:
         spec = WORKLOADS[args.workload]

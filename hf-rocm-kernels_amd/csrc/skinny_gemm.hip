@@ -768,7 +768,7 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
 }
 
 static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p, bool packed = false) {
-    if (swiglu && p->wn != 0 && p->wn != -2) return HFRK_INVALID_CONFIG;  // the fused epilogue: wave-stream and row-split kernels
+    if (swiglu && p->wn != 0 && p->wn != -2 && p->wn != -1) return HFRK_INVALID_CONFIG;  // the workgroup kernel has no fused epilogue
     if (p->wn == -2) {  // row-split decomposition: wk = matrix tiles per chunk, ch = activation loads
         if (packed) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
         if (swiglu && p->wk != 2) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows
@@ -790,6 +790,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
         if (p->m_tiles != want.m_tiles || p->ch != 0 || p->panels != want.panels || p->slabs != want.slabs ||
             p->lds_bytes != want.lds_bytes)
             return HFRK_INVALID_CONFIG;
+        if (swiglu && (want.slabs != 1 || p->wk > 2)) return HFRK_INVALID_CONFIG;  // gate and up sums meet inside one workgroup
         if ((long)want.panels * want.slabs * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;
         return HFRK_SUCCESS;
     }
@@ -913,7 +914,8 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     if ((sa_stride != 0 && sa_stride != 1) || (sb_stride != 0 && sb_stride != 1)) return HFRK_BAD_SHAPE;
     if (epilogue != HFRK_EPILOGUE_NONE && epilogue != HFRK_EPILOGUE_SWIGLU) return HFRK_INVALID_CONFIG;
     const bool swiglu = epilogue == HFRK_EPILOGUE_SWIGLU;
-    if (swiglu && (!out_scale || base || m > 16 || n % 32 != 0)) return HFRK_BAD_SHAPE;
+    // SwiGLU epilogue: up to 16 rows in the wave-stream / row-split kernels; above, in the K-split kernel when one window covers K
+    if (swiglu && (!out_scale || base || n % 32 != 0 || (m > 16 && k != 2048 && k != 4096))) return HFRK_BAD_SHAPE;
     // every offset the kernel forms, including rows of the last (padded) panel, must stay below 2^31
     if (((long)n + 128) * b_stride + k >= (1L << 31) || (long)m * k >= (1L << 31)) return HFRK_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15 || (b_stride & 15)) return HFRK_BAD_ALIGNMENT;
@@ -946,7 +948,9 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         if (rc != HFRK_SUCCESS) return rc;
     } else {
         int rc;
-        if (swiglu && !packed && make_rows_plan(m, n / 2, k, &p) == HFRK_SUCCESS) {
+        if (swiglu && m > 16) {
+            rc = make_ksplit_plan(m, n / 2, k, &p);  // tiles of 16 output columns; a gate and an up pass per tile
+        } else if (swiglu && !packed && make_rows_plan(m, n / 2, k, &p) == HFRK_SUCCESS) {
             // bands of output columns; every chunk holds the gate rows and the up rows of up to 16 of them
             rc = fill_rows_plan(m, n / 2, k, 2, p.grid, &p);
         } else if (swiglu) {
@@ -1030,7 +1034,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         return launch_rows_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     }
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
-    if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, p.lds_bytes, stream);
+    if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, swiglu, p.lds_bytes, stream);
     switch (p.m_tiles) {
         case 1: return launch_mt<1>(args, p, stream);
         case 2: return launch_mt<2>(args, p, stream);

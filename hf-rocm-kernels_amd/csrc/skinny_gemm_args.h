@@ -66,7 +66,9 @@ constexpr bool rows_variant_exists(int act_loads, int row_tiles) {
 
 // K-split kernel (skinny_gemm_ksplit.hip): the 8 waves of a workgroup split a K window of 8*wave_k bytes
 // (wave_k = 256, 512, or 1024 with m_tiles <= 2), activations in registers.  Needs k % (8*wave_k) == 0.
-int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, int lds_bytes, hipStream_t stream);
+// swiglu: gate rows [0, n/2), up rows [n/2, n); one window must cover K (wave_k = k / 8 = 256 or 512); panels counts the tiles of
+// 16 output columns (n / 32), D is fp8 [m, n/2]
+int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, bool swiglu, int lds_bytes, hipStream_t stream);
 constexpr bool ksplit_variant_exists(int m_tiles, int wave_k) {
     return m_tiles >= 1 && (((wave_k == 256 || wave_k == 512) && m_tiles <= 4) || (wave_k == 1024 && m_tiles <= 2));
 }

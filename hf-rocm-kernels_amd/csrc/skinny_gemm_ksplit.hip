@@ -26,9 +26,15 @@ namespace hfrk {
 // PACKED: the weight is in the pre-packed layout (pack_weight.hip), chunk (tile, kc) at (tile * k/256 + kc) * 4096 in
 // MFMA operand order: a wave's piece of a unit is KW/256 contiguous chunks, the loaded registers are the operands,
 // and each chunk of the next unit is requested as soon as the MFMAs of the current one have taken its registers.
-template <int MT, int KW, bool PACKED>
+// SWIGLU: the weight is a gate_up projection (gate rows [0, n/2), up rows [n/2, n)) and one window covers K.  A unit
+// is then a tile of 16 output columns, worked as two passes of the loop body: the gate tile t, whose finished sums the
+// waves 0..MT-1 keep in registers, then the up tile t + n/32, after which they store
+// e4m3fn(silu(gate) * up / out_scale) into D [m, n/2] instead of the two 16-bit projections -- the SwiGLU kernel of
+// csrc/op_src/swiglu/swiglu_vectorized.cu:27-97 as the GEMM's epilogue, here for 17..64 rows.
+template <int MT, int KW, bool PACKED, bool SWIGLU>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const GemmArgs a) {
     constexpr uint32_t kOutOfRange = 0x80000000u;
+    constexpr int PASSES = SWIGLU ? 2 : 1;
     constexpr int kCoherent = 17;     // sc0 | sc1
     constexpr int KCH = KW / 256;     // 256-byte column chunks of a wave's weight piece
     constexpr int KST = KW / 128;     // MFMA K steps per unit
@@ -45,8 +51,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
 
     // ---- this workgroup's units (u = window * T + tile; 32-bit, the host checks (grid + 1) * units < 2^31) ---------
     const int G = a.grid;
-    const int T = a.panels;  // 16-row tiles
-    const int S = a.slabs;   // windows
+    const int T = a.panels;  // 16-row tiles (SWIGLU: tiles of 16 output columns, T = n / 32)
+    const int S = a.slabs;   // windows (SWIGLU: 1)
     const int b = blockIdx.x;
     const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;  // XCD x owns logical ids [x*G/8, (x+1)*G/8)
     const uint32_t uq = (uint32_t)a.chunks_q, ur = (uint32_t)a.chunks_r;  // units / G, units % G
@@ -55,25 +61,27 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     int win = (int)(u0 / (uint32_t)T);
     int tile = (int)(u0 - (uint32_t)win * (uint32_t)T);
 
-    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, PACKED ? (uint32_t)T * (uint32_t)a.k * 16u
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, PACKED ? (uint32_t)(PASSES * T) * (uint32_t)a.k * 16u
                                                                 : (uint32_t)(a.n - 1) * (uint32_t)a.b_stride + (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(a.A, (uint32_t)a.m * (uint32_t)a.k);
     const __amdgpu_buffer_rsrc_t ws_rsrc = make_rsrc(a.ws, a.ws_bytes);
-    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)a.n * 2u);
+    const int n_out = SWIGLU ? (a.n >> 1) : a.n;  // columns of D
+    const __amdgpu_buffer_rsrc_t d_rsrc = make_rsrc(a.D, (uint32_t)a.m * (uint32_t)n_out * (SWIGLU ? 1u : 2u));
     const __amdgpu_buffer_rsrc_t base_rsrc = make_rsrc(a.base, a.base ? (uint32_t)a.m * (uint32_t)a.n * 2u : 0u);
     const __amdgpu_buffer_rsrc_t sb_rsrc = make_rsrc(a.scale_b, a.scale_b ? (uint32_t)a.n * 4u : 0u);
-    const bool accumulate = a.base != nullptr;
+    const bool accumulate = !SWIGLU && a.base != nullptr;
     const bool per_channel = a.scale_b && a.sb_stride;
-    const bool vec = (a.n & 3) == 0;
+    const bool vec = SWIGLU || (a.n & 3) == 0;
 
     // ---- weight stream: load t of column chunk c brings rows 4t + lg, bytes c*256 + li*16 .. +16 of the wave's piece --
     const uint32_t w_lane_off = (uint32_t)lg * (uint32_t)a.b_stride + (uint32_t)wv * KW + (uint32_t)li * 16u;
     v4i wq[KCH][4];
     int itile = tile, iwin = win;  // unit being requested
+    int ipass = 0;                 // SWIGLU: 0 = its gate tile, 1 = its up tile
     // column chunk c of the wave's piece of unit (itile, iwin); `base` is the unit's row-major offset
     auto issue_chunk = [&](int c, uint32_t base) __attribute__((always_inline)) {
         if constexpr (PACKED) {
-            const uint32_t chunk = (uint32_t)itile * ((uint32_t)a.k >> 8) + ((uint32_t)iwin * 8u + (uint32_t)wv) * KCH + (uint32_t)c;
+            const uint32_t chunk = (uint32_t)(itile + ipass * T) * ((uint32_t)a.k >> 8) + ((uint32_t)iwin * 8u + (uint32_t)wv) * KCH + (uint32_t)c;
 #pragma unroll
             for (int t = 0; t < 4; ++t)
                 wq[c][t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(chunk * (uint32_t)kTileBytes + (uint32_t)t * 1024u + (uint32_t)lane * 16u), 0, 2 /* nt */);
@@ -84,7 +92,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
         }
     };
     auto issue_unit = [&]() __attribute__((always_inline)) {
-        const uint32_t base = (uint32_t)itile * 16u * (uint32_t)a.b_stride + (uint32_t)iwin * (8u * KW);
+        const uint32_t base = (uint32_t)(itile + ipass * T) * 16u * (uint32_t)a.b_stride + (uint32_t)iwin * (8u * KW);
 #pragma unroll
         for (int c = 0; c < KCH; ++c) issue_chunk(c, base);
     };
@@ -181,6 +189,34 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
         }
     };
 
+    // SWIGLU: gate and up sums of output columns n0 .. n0+3 (n0 = t*16 + 4*lg) of row mt*16 + li, each rounded to the
+    // 16-bit dtype the unfused chain stores between its two kernels, then silu(gate) * up / out_scale as four fp8
+    float inv_out_scale = 1.0f;
+    if constexpr (SWIGLU) {
+        const float os = a.out_scale[0];
+        inv_out_scale = os != 0.f ? 1.0f / os : 1.0f;
+    }
+    auto epilogue_swiglu = [&](int t, int mt, v4f gate, v4f up) __attribute__((always_inline)) {
+        const int n0 = t * 16 + 4 * lg;
+        const int mrow = mt * 16 + li;
+        const bool live = mrow < a.m && n0 < n_out;
+        const v4f sbg = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (live && per_channel) ? n0 * 4 : (int)kOutOfRange, 0, 0));
+        const v4f sbu = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (live && per_channel) ? (n_out + n0) * 4 : (int)kOutOfRange, 0, 0));
+        const float sam = mt == 0 ? sa[0] : mt == 1 ? sa[MT > 1 ? 1 : 0] : mt == 2 ? sa[MT > 2 ? 2 : 0] : sa[MT > 3 ? 3 : 0];
+        float y[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float g = gate[v] * (sam * (per_channel ? sbg[v] : 1.0f));
+            float u = up[v] * (sam * (per_channel ? sbu[v] : 1.0f));
+            g = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(g)) : load16<HFRK_F16>(store16<HFRK_F16>(g));
+            u = a.d_dtype == HFRK_BF16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(u)) : load16<HFRK_F16>(store16<HFRK_F16>(u));
+            y[v] = silu_mul(g, u, inv_out_scale);
+        }
+        uint32_t packed = cvt_pk_fp8(y[0], y[1], 0u, false);
+        packed = cvt_pk_fp8(y[2], y[3], packed, true);
+        __builtin_amdgcn_raw_buffer_store_b32((int)packed, d_rsrc, live ? (int)((uint32_t)mrow * (uint32_t)n_out + (uint32_t)n0) : (int)kOutOfRange, 0, 0);
+    };
+
     // Several windows (S > 1): a unit's share of its tile goes to the workspace and an arrival counter decides who adds
     // the shares.  Store, acknowledgement, counter round trip and the verdict are spread over two units so that none of
     // them is waited for where it was issued: the share is stored at the end of unit i, acknowledged and counted at the
@@ -220,8 +256,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     };
 
     // ---- unit loop ----------------------------------------------------------------------------------------------------
+    v4f gate_sum = v4f{0.f, 0.f, 0.f, 0.f};  // SWIGLU, waves 0..MT-1: the gate tile's sums, kept over the up tile's pass
 #pragma unroll 1
-    for (int i = 0; i < count; ++i) {
+    for (int i = 0; i < PASSES * count; ++i) {
         if constexpr (!PACKED) {
 #pragma unroll
             for (int c = 0; c < KCH; ++c)
@@ -231,10 +268,15 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
         if constexpr (kDeferred) {
             if (S > 1 && wv < MT && stored_tile >= 0) count_arrival();
         }
-        const bool more = i + 1 < count;
+        const bool more = i + 1 < PASSES * count;
         bool new_window = false;
         if (more) {  // row-major: registers are free again, request the next unit before the LDS reads and MFMAs
-            if (++itile == T) { itile = 0; ++iwin; new_window = true; }
+            if (SWIGLU && ipass == 0) {
+                ipass = 1;  // the same columns' up tile
+            } else {
+                ipass = 0;
+                if (++itile == T) { itile = 0; ++iwin; new_window = true; }
+            }
             if constexpr (!PACKED) issue_unit();
         }
         if constexpr (!PACKED) {
@@ -299,6 +341,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
                     count_arrival();
                     settle();
                 }
+            } else if constexpr (SWIGLU) {
+                if ((i & 1) == 0) gate_sum = sum;
+                else epilogue_swiglu(tile, wv, gate_sum, sum);
             } else {
                 epilogue(tile, wv, sum);
             }
@@ -320,9 +365,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_ksplit_kernel(const 
     }
 }
 
-template <int MT, int KW, bool PACKED>
+template <int MT, int KW, bool PACKED, bool SWIGLU>
 static int launch_ksplit_packing(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_ksplit_kernel<MT, KW, PACKED>;
+    auto kern = skinny_gemm_ksplit_kernel<MT, KW, PACKED, SWIGLU>;
     static bool attr_done[64] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -336,21 +381,28 @@ static int launch_ksplit_packing(const GemmArgs& args, int lds_bytes, hipStream_
 }
 
 template <int MT, int KW>
-static int launch_ksplit_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    return args.packed ? launch_ksplit_packing<MT, KW, true>(args, lds_bytes, stream)
-                       : launch_ksplit_packing<MT, KW, false>(args, lds_bytes, stream);
+static int launch_ksplit_one(const GemmArgs& args, bool swiglu, int lds_bytes, hipStream_t stream) {
+    if constexpr (KW <= 512) {  // the SwiGLU epilogue: one window of 2048 or 4096 bytes covers K
+        if (swiglu)
+            return args.packed ? launch_ksplit_packing<MT, KW, true, true>(args, lds_bytes, stream)
+                               : launch_ksplit_packing<MT, KW, false, true>(args, lds_bytes, stream);
+    }
+    if (swiglu) return HFRK_INVALID_CONFIG;
+    return args.packed ? launch_ksplit_packing<MT, KW, true, false>(args, lds_bytes, stream)
+                       : launch_ksplit_packing<MT, KW, false, false>(args, lds_bytes, stream);
 }
 
-int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, int lds_bytes, hipStream_t stream) {
+int launch_ksplit_kernel(const GemmArgs& args, int m_tiles, int wave_k, bool swiglu, int lds_bytes, hipStream_t stream) {
     if (lds_bytes != ksplit_lds_bytes(m_tiles, wave_k)) return HFRK_INVALID_CONFIG;
     if (!ksplit_variant_exists(m_tiles, wave_k)) return HFRK_INVALID_CONFIG;
+    if (swiglu && args.slabs != 1) return HFRK_INVALID_CONFIG;
 #define HFRK_KSPLIT_CASE(MT_)                                                                          \
     case MT_:                                                                                          \
-        return wave_k == 256 ? launch_ksplit_one<MT_, 256>(args, lds_bytes, stream)                    \
-                             : launch_ksplit_one<MT_, 512>(args, lds_bytes, stream);
+        return wave_k == 256 ? launch_ksplit_one<MT_, 256>(args, swiglu, lds_bytes, stream)            \
+                             : launch_ksplit_one<MT_, 512>(args, swiglu, lds_bytes, stream);
     if (wave_k == 1024) {  // 16*MT rows x 1 KB of activations per wave: registers allow two tiles
-        return m_tiles == 1 ? launch_ksplit_one<1, 1024>(args, lds_bytes, stream)
-                            : launch_ksplit_one<2, 1024>(args, lds_bytes, stream);
+        return m_tiles == 1 ? launch_ksplit_one<1, 1024>(args, swiglu, lds_bytes, stream)
+                            : launch_ksplit_one<2, 1024>(args, swiglu, lds_bytes, stream);
     }
     switch (m_tiles) {
         HFRK_KSPLIT_CASE(1)

@@ -219,12 +219,13 @@ def skinny_gemm_swiglu(
     """gate_up projection and SwiGLU in one launch: with [gate | up] = scale_a * scale_b * (skinny_a @ gate_up_weight)
     rounded to `intermediate_dtype`, returns float8_e4m3fn(silu(gate) * up / out_scale) of shape (m, n/2) -- what
     `skinny_gemm` followed by `swiglu` produces, without the (m, n) intermediate and the second launch.
-    For m <= 16 and n % 32 == 0; other shapes run the two kernels."""
+    One launch for n % 32 == 0 and m <= 16, or m <= 64 on k = 2048 / 4096 (`hfrk_skinny_gemm_fused`'s conditions); other
+    shapes run the two kernels."""
     m, n = skinny_a.size(0), gate_up_weight.size(1)
     assert n % 2 == 0, f"Expected an even number of gate_up columns but got {n}"
     assert intermediate_dtype in _OUT_DTYPES, f"Expected one of {_OUT_DTYPES} but got {intermediate_dtype = }"
     assert out_scale.numel() == 1 and out_scale.dtype == torch.float32, "Expected out_scale to be one float32"
-    if m > 16 or n % 32 != 0:
+    if n % 32 != 0 or (m > 16 and skinny_a.size(1) not in (2048, 4096)):
         from ..swiglu import swiglu
         gate_up = skinny_gemm_scaled(skinny_a, gate_up_weight, scale_a,
                                      scale_b if scale_b is not None else torch.ones(1, device=skinny_a.device),

@@ -359,7 +359,8 @@ def _swiglu_oracle(a, w, sa, sb, out_scale, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("m,n,k", [(1, 512, 1024), (5, 2080, 512), (8, 28672, 4096), (13, 1024, 2048), (16, 28672, 4096),
-                                   (16, 64, 256)])
+                                   (16, 64, 256), (17, 1024, 4096), (32, 28672, 4096), (40, 4160, 2048), (64, 2048, 2048),
+                                   (64, 28672, 4096)])
 def test_swiglu_epilogue_matches_the_two_kernel_chain(m, n, k, per_channel, dtype):
     """One launch (GEMM with SwiGLU epilogue) against GEMM -> 16-bit -> swiglu, on the device and in the oracle.
     The two device paths may sum K in a different order, so a 16-bit projection can differ by one rounding and an
@@ -396,13 +397,25 @@ def test_swiglu_epilogue_limits_and_fallback():
     assert lib.hfrk_skinny_gemm_fused(*bad) == _capi.BAD_SHAPE                # base with the SwiGLU epilogue
     bad = list(args(8, 512)); bad[14] = 7
     assert lib.hfrk_skinny_gemm_fused(*bad) == _capi.INVALID_CONFIG
-    # the Python wrapper falls back to GEMM + swiglu above 16 rows
+    # above 16 rows the epilogue exists where one K-split window covers k (2048, 4096): k = 512 is not among them, and the
+    # K-split kernel takes no plan that cuts k into several windows with it
+    a4, w4, sa4, sw4 = generate_llama_gemm_data(32, 512, 4096, seed=4)
+    out4 = torch.empty(32, 256, dtype=torch.float8_e4m3fn).cuda()
+    args4 = (a4.data_ptr(), w4.data_ptr(), out4.data_ptr(), None, sa4.data_ptr(), 0, sw4.data_ptr(), 0, out_scale.data_ptr(),
+             32, 512, 4096, 4096, _capi.BF16, _capi.EPILOGUE_SWIGLU)
+    assert lib.hfrk_skinny_gemm_fused(*args4, None, None) == _capi.SUCCESS
+    windows = _capi.GemmPlan(2, -1, 1, 0, 32, 16, 2, 8 * 4096 + 16 * 2 * 1024)   # 256 bytes per wave: two windows
+    assert lib.hfrk_skinny_gemm_fused(*args4, ctypes.byref(windows), None) == _capi.INVALID_CONFIG
+    workgroup = _capi.GemmPlan(2, 4, 2, 1, 32, 4, 8, 8 * 4096 + 2 * 16 * 2 * 512)
+    assert lib.hfrk_skinny_gemm_fused(*args4, ctypes.byref(workgroup), None) == _capi.INVALID_CONFIG
+    torch.cuda.synchronize()
+    # the Python wrapper falls back to GEMM + swiglu where the epilogue does not exist
     got = skinny_gemm_swiglu(a, w, sa, sw, out_scale)
     ref, tol = _swiglu_oracle(a, w, sa, sw, out_scale, torch.bfloat16)
     assert ((got.cpu().float() - ref.float()).abs() <= tol).all()
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 1024, 2048), (16, 6144, 1024), (3, 2080 * 2, 512)])
+@pytest.mark.parametrize("m,n,k", [(8, 1024, 2048), (16, 6144, 1024), (3, 2080 * 2, 512), (40, 2080 * 2, 4096), (64, 1024, 2048)])
 def test_swiglu_epilogue_under_every_split(m, n, k):
     """Forced plans: grids that cut (gate, up) tile pairs between waves and between workgroups in different places."""
     from hf_rocm_kernels import _capi
@@ -412,6 +425,21 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
     out_scale = torch.tensor([8.0 / 448], dtype=torch.float32).cuda()
     ref, tol = _swiglu_oracle(a, w, sa, sw, out_scale, torch.bfloat16)
     ma, kc, groups = (m + 3) // 4, k // 256, (n // 2) // 16
+    if k in (2048, 4096):  # K-split plans: one window covers k, the workgroup's 8 waves split it
+        mt, wave_k = (m + 15) // 16, k // 8
+        for grid in sorted({min(g, groups) for g in (256, 200, 7, 1)}):
+            plan = _capi.GemmPlan(mt, -1, wave_k // 256, 0, grid, groups, 1, 8 * (wave_k // 256) * 4096 + 16 * mt * 1024)
+            out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
+            st = lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                                            out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
+                                            ctypes.byref(plan), torch.cuda.current_stream().cuda_stream)
+            assert st == 0, ("k-split", grid, st)
+            torch.cuda.synchronize()
+            f = out.cpu().float()
+            assert not f.isnan().any(), ("k-split", grid)
+            assert ((f - ref.float()).abs() <= tol).all(), ("k-split", grid)
+    if m > 16:
+        return
     for grid in sorted({min(g, groups * kc) for g in (256, 200, 64, 7, 1)}):
         plan = _capi.GemmPlan((ma + 3) // 4, 0, 2, ma, grid, groups, kc, 8 * (2 + (ma + 3) // 4) * 4096)
         out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)

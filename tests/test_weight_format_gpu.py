@@ -181,7 +181,8 @@ def test_float16_output_and_accumulation_on_a_packed_weight(m, n, k):
     check_against_oracle(got, a, b, sa, sw, base=base)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 1024, 1024), (8, 28672, 4096), (16, 2080, 2048), (5, 96, 256)])
+@pytest.mark.parametrize("m,n,k", [(1, 1024, 1024), (8, 28672, 4096), (16, 2080, 2048), (5, 96, 256), (40, 2080, 2048),
+                                   (64, 1024, 4096)])
 def test_swiglu_epilogue_on_a_packed_weight_equals_the_row_major_result(m, n, k):
     from hf_rocm_kernels import _capi
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
