@@ -56,8 +56,8 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
 
 HBM_PEAK_GBPS = 8000.0
 # Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0097 x the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55227698}
+# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0094 x the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55216472}
 CALIBRATION_COPY_BYTES = 256 << 20
 
 WORKLOADS = {
@@ -198,9 +198,16 @@ def capture_gemm_steps(torch, spec, call):
     return graphs, outs
 
 
-def time_graph(torch, g, calls, reps):
-    for _ in range(3):
+def time_graph(torch, g, calls, reps, warm_ms=10.0):
+    # Building a graph leaves the GPU idle for milliseconds and its clocks come down: replay for `warm_ms` first, so that a
+    # short graph (10 launches of 15 us) is timed in the same state as the pre-rolled timed region.
+    t0 = time.perf_counter()
+    n = 0
+    while n < 3 or (time.perf_counter() - t0) * 1e3 < warm_ms:
         g.replay()
+        n += 1
+        if n % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     ts = []
     for _ in range(reps):
@@ -215,8 +222,9 @@ def time_graph(torch, g, calls, reps):
 
 
 def time_gemm_cases(torch, spec, call, weights, reps=40):
-    """Per-(shape, M): time from a graph of one launch per weight copy (HBM-cold) and from a graph of 32 launches on
-    one copy (cache-hot: what the 256 MB Infinity Cache holds is not re-fetched from HBM)."""
+    """Per-(shape, M): time from a graph that walks the weight copies in rotation, at least 32 launches (HBM-cold: every
+    shape's copies add up to several times the 256 MB Infinity Cache), and from a graph of 32 launches on one copy
+    (cache-hot: what the Infinity Cache holds is not re-fetched from HBM)."""
     rows = []
     stream = torch.cuda.Stream()
     n_scales = lambda m, n: (m + n) if spec["scaled"] else 1
@@ -227,15 +235,17 @@ def time_gemm_cases(torch, spec, call, weights, reps=40):
             with torch.cuda.stream(stream):
                 call(name, n, k, m, 0, out)
             torch.cuda.synchronize()
+            rounds = -(-32 // copies)  # at least 32 launches per graph: the graph's own start-up is then a small share of a replay
             cold = torch.cuda.CUDAGraph()
             with torch.cuda.graph(cold, stream=stream):
-                for ci in range(copies):
-                    call(name, n, k, m, ci, out)
+                for _ in range(rounds):
+                    for ci in range(copies):
+                        call(name, n, k, m, ci, out)
             hot = torch.cuda.CUDAGraph()
             with torch.cuda.graph(hot, stream=stream):
                 for _ in range(32):
                     call(name, n, k, m, 0, out)
-            us, std = time_graph(torch, cold, copies, reps)
+            us, std = time_graph(torch, cold, copies * rounds, reps)
             us_hot, _ = time_graph(torch, hot, 32, reps)
             gbps = gemm_bytes(m, n, k, n_scales(m, n)) / us / 1e3
             rows.append({"shape": name, "n": n, "k": k, "m": m, "us_per_call": round(us, 3), "us_std": round(std, 3),
