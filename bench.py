@@ -286,7 +286,7 @@ def cpu_baseline_gemm(torch, spec, budget_s):
 
     one_pass()  # warm-up
     times, spent = [], 0.0
-    while len(times) < 2 or (spent < budget_s and len(times) < 9):
+    while len(times) < 2 or (spent < budget_s and len(times) < 31):
         t = one_pass()
         times.append(t)
         spent += t
@@ -404,7 +404,7 @@ def cpu_baseline_mlp(torch, budget_s):
 
     one_pass()
     times, spent = [], 0.0
-    while len(times) < 2 or (spent < budget_s and len(times) < 9):
+    while len(times) < 2 or (spent < budget_s and len(times) < 31):
         t = one_pass()
         times.append(t)
         spent += t

@@ -360,7 +360,7 @@ def _swiglu_oracle(a, w, sa, sb, out_scale, dtype):
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("m,n,k", [(1, 512, 1024), (5, 2080, 512), (8, 28672, 4096), (13, 1024, 2048), (16, 28672, 4096),
                                    (16, 64, 256), (17, 1024, 4096), (32, 28672, 4096), (40, 4160, 2048), (64, 2048, 2048),
-                                   (64, 28672, 4096)])
+                                   (64, 28672, 4096), (8, 1024, 640), (3, 4160, 4096 + 128)])
 def test_swiglu_epilogue_matches_the_two_kernel_chain(m, n, k, per_channel, dtype):
     """One launch (GEMM with SwiGLU epilogue) against GEMM -> 16-bit -> swiglu, on the device and in the oracle.
     The two device paths may sum K in a different order, so a 16-bit projection can differ by one rounding and an
