@@ -16,6 +16,7 @@ Other workloads, same method, for the remaining configurations:
               (`skinny_gemm_scaled`, activation rows 1 and M-1 drawn 20x larger)
   mlp         the decoder MLP sub-block (`llama_mlp_combined_ops`: residual RMSNorm -> gate_up GEMM -> SwiGLU ->
               down GEMM, output added to the residual), hidden 4096, M in {1, 8, 16}: 3 blocks = 12 launches per step
+  mlp-rms     the fused block with the RMSNorm as the gate_up GEMM's prologue: two launches up to 8 rows
   mlp-fused   the same block in three launches: RMSNorm, gate_up GEMM with SwiGLU epilogue, down GEMM reading the
               residual as its addend (`llama_mlp_combined_ops(..., fused=True)`)
   pack        the step before the path: the four Llama-3-8B weights packed into the load format from float8_e4m3fn,
@@ -330,7 +331,7 @@ def make_mlp_inputs(torch, packed=False):
     return copies, acts, rms_w, s_in, s_mid
 
 
-def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused):
+def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused, rms_prologue=False):
     from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
     out_scales = [((s_in * sgu).contiguous(), (s_mid * sd).contiguous()) for _, sgu, _, sd in copies]
 
@@ -338,7 +339,7 @@ def mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused):
         wgu, _, wd, _ = copies[ci]
         x, res = acts[m]
         return llama_mlp_combined_ops(x, res, rms_w, MLP["eps"], wgu, s_in, out_scales[ci][0], wd, s_mid,
-                                      out_scales[ci][1], add_residual=True, fused=fused)
+                                      out_scales[ci][1], add_residual=True, fused=fused, rms_prologue=rms_prologue)
     return call
 
 
@@ -575,7 +576,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "pack", "floor"], default="llama3-8b")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "mlp-rms", "pack", "floor"], default="llama3-8b")
     ap.add_argument("--detail", action="store_true", help="kept for older command lines: the per-case table is on by default")
     ap.add_argument("--no-cases", action="store_true", help="skip the per-case table after the timed steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -609,11 +610,12 @@ def main():
         if args.workload in WORKLOADS:
             WORKLOADS[args.workload]["ms"] = rows
             WORKLOADS[args.workload]["text"] += " [--ms " + args.ms + "]"
-    is_mlp = args.workload in ("mlp", "mlp-fused")
+    is_mlp = args.workload in ("mlp", "mlp-fused", "mlp-rms")
     if is_mlp:
-        fused = args.workload == "mlp-fused"
+        fused = args.workload in ("mlp-fused", "mlp-rms")
+        two = args.workload == "mlp-rms"  # RMSNorm as the gate_up GEMM's prologue: two launches where the library has it (up to 8 rows)
         copies, acts, rms_w, s_in, s_mid = make_mlp_inputs(torch, args.packed)
-        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused)
+        call = mlp_caller(torch, copies, acts, rms_w, s_in, s_mid, fused, two)
         graphs, keep = capture_mlp_steps(torch, call)
         step_bytes = sum(mlp_block_bytes(m) for m in MLP["ms"])
         calls, text, metric = (3 if fused else 4) * len(MLP["ms"]), MLP["text"], MLP["metric"]
@@ -621,6 +623,12 @@ def main():
             text = text.replace("3 blocks = 12 launches", "fused into 3 launches per block: 3 blocks = 9 launches")
         kernel = ("residual_rms_vec_kernel + skinny_gemm_rows_kernel<MA,2,swiglu> + skinny_gemm_rows_kernel" if fused else
                   "residual_rms_vec_kernel + skinny_gemm_rows_kernel + swiglu_vec_kernel + skinny_gemm_rows_kernel")
+        if two:
+            small = sum(1 for m in MLP["ms"] if m <= 8)
+            calls = 2 * small + 3 * (len(MLP["ms"]) - small)
+            text = text.replace("fused into 3 launches per block: 3 blocks = 9 launches",
+                                "2 launches per block up to 8 rows (RMSNorm as the gate_up GEMM's prologue), 3 above: %d launches" % calls)
+            kernel = "skinny_gemm_rows_kernel<MA,2,swiglu,rms> + skinny_gemm_rows_kernel (up to 8 rows; the three-launch kernels above)"
         if args.packed:  # the packed format is read by the wave-stream kernel
             kernel = kernel.replace("rows_kernel", "stream_kernel")
         n_copies = MLP["cycle"]

@@ -85,6 +85,49 @@ __device__ __forceinline__ float silu_mul(float g, float u, float inv_scale) {
     return g * __builtin_amdgcn_rcpf(1.0f + e) * u * inv_scale;
 }
 
+// Sum over the 64 lanes of a wave (xor butterfly): every lane returns the same bits.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// The two per-piece steps of the residual RMSNorm on 8 elements (16 bytes) of a row, shared by the stand-alone kernel
+// (residual_rms.hip) and the GEMM's RMSNorm prologue (skinny_gemm_rows.hip) so that both produce the same bits:
+//   z = round16(float(input) + float(residual)), ssq += float(z)^2 in element order;
+//   fp8 = e4m3fn(clamp(float(z) * norm * float(weight) * inv_scale, +-448)).
+template <int DT>
+__device__ __forceinline__ uint4 rms_add_square(uint4 a, uint4 r, float& ssq) {
+    const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, rw[4] = {r.x, r.y, r.z, r.w};
+    uint32_t zw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint16_t lo = store16<DT>(load16<DT>((uint16_t)(aw[j] & 0xffff)) + load16<DT>((uint16_t)(rw[j] & 0xffff)));
+        const uint16_t hi = store16<DT>(load16<DT>((uint16_t)(aw[j] >> 16)) + load16<DT>((uint16_t)(rw[j] >> 16)));
+        const float fl = load16<DT>(lo), fh = load16<DT>(hi);
+        ssq += fl * fl;
+        ssq += fh * fh;
+        zw[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+    return make_uint4(zw[0], zw[1], zw[2], zw[3]);
+}
+
+template <int DT>
+__device__ __forceinline__ uint2 rms_scale_to_fp8(uint4 z, uint4 w, float norm, float inv_scale) {
+    const uint32_t zw[4] = {z.x, z.y, z.z, z.w}, ww[4] = {w.x, w.y, w.z, w.w};
+    float y[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        y[2 * j] = load16<DT>((uint16_t)(zw[j] & 0xffff)) * norm * load16<DT>((uint16_t)(ww[j] & 0xffff)) * inv_scale;
+        y[2 * j + 1] = load16<DT>((uint16_t)(zw[j] >> 16)) * norm * load16<DT>((uint16_t)(ww[j] >> 16)) * inv_scale;
+    }
+    uint32_t p0 = cvt_pk_fp8(y[0], y[1], 0u, false);
+    p0 = cvt_pk_fp8(y[2], y[3], p0, true);
+    uint32_t p1 = cvt_pk_fp8(y[4], y[5], 0u, false);
+    p1 = cvt_pk_fp8(y[6], y[7], p1, true);
+    return make_uint2(p0, p1);
+}
+
 // Raw buffer resource over [base, base+bytes): loads beyond `bytes` return zero instead of faulting.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);

@@ -18,12 +18,6 @@ namespace hfrk {
 
 constexpr int kRmsMaxThreads = 1024;
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
 // Sum over the workgroup; every thread returns the same bits.
 __device__ __forceinline__ float block_sum(float v, float* red) {
     v = wave_sum(v);
@@ -75,18 +69,7 @@ __global__ void __launch_bounds__(kRmsMaxThreads) residual_rms_vec_kernel(
         if (v < nvec) {
             const uint4 a = reinterpret_cast<const uint4*>(input + row_off)[v];
             const uint4 r = reinterpret_cast<const uint4*>(residual + row_off)[v];
-            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, rw[4] = {r.x, r.y, r.z, r.w};
-            uint32_t zw[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint16_t lo = store16<DT>(load16<DT>((uint16_t)(aw[j] & 0xffff)) + load16<DT>((uint16_t)(rw[j] & 0xffff)));
-                const uint16_t hi = store16<DT>(load16<DT>((uint16_t)(aw[j] >> 16)) + load16<DT>((uint16_t)(rw[j] >> 16)));
-                const float fl = load16<DT>(lo), fh = load16<DT>(hi);
-                ssq += fl * fl;
-                ssq += fh * fh;
-                zw[j] = (uint32_t)lo | ((uint32_t)hi << 16);
-            }
-            z[it] = make_uint4(zw[0], zw[1], zw[2], zw[3]);
+            z[it] = rms_add_square<DT>(a, r, ssq);
             reinterpret_cast<uint4*>(residual + row_off)[v] = z[it];
         }
     }
@@ -101,17 +84,7 @@ __global__ void __launch_bounds__(kRmsMaxThreads) residual_rms_vec_kernel(
             const uint4 w = wreg[it];
             const uint32_t zw[4] = {z[it].x, z[it].y, z[it].z, z[it].w}, ww[4] = {w.x, w.y, w.z, w.w};
             if constexpr (FP8_OUT) {
-                float y[8];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    y[2 * j] = load16<DT>((uint16_t)(zw[j] & 0xffff)) * norm * load16<DT>((uint16_t)(ww[j] & 0xffff)) * inv_scale;
-                    y[2 * j + 1] = load16<DT>((uint16_t)(zw[j] >> 16)) * norm * load16<DT>((uint16_t)(ww[j] >> 16)) * inv_scale;
-                }
-                uint32_t p0 = cvt_pk_fp8(y[0], y[1], 0u, false);
-                p0 = cvt_pk_fp8(y[2], y[3], p0, true);
-                uint32_t p1 = cvt_pk_fp8(y[4], y[5], 0u, false);
-                p1 = cvt_pk_fp8(y[6], y[7], p1, true);
-                reinterpret_cast<uint2*>(static_cast<uint8_t*>(output) + row_off)[v] = make_uint2(p0, p1);
+                reinterpret_cast<uint2*>(static_cast<uint8_t*>(output) + row_off)[v] = rms_scale_to_fp8<DT>(z[it], w, norm, inv_scale);
             } else {
                 uint32_t ow[4];
 #pragma unroll

@@ -902,14 +902,36 @@ static long plan_counters(const hfrk_gemm_plan& p) { return p.wn == -2 ? 0 : p.w
 
 // D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
 // use_static: partial sums and counters go to this device's `scratch` array instead of the stream's workspace.
+// rms: the activations are not read from A but built by the kernel's RMSNorm prologue from these 16-bit tensors.
+struct RmsPrologue {
+    const void* input;
+    const void* residual;
+    void* residual_out;
+    const void* weight;
+    const float* act_scale;
+    float epsilon;
+    int dtype;
+};
 static int gemm_launch(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
                        const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k, int b_stride,
                        int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream, bool packed = false,
-                       bool use_static = false) {
+                       bool use_static = false, const RmsPrologue* rms = nullptr) {
     if (packed) b_stride = k;
     if (m < 1 || m > HFRK_GEMM_MAX_M || n < 1 || k < 1 || b_stride < k) return HFRK_BAD_SHAPE;
     if (k % 16 != 0 || (packed && k % 256 != 0)) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (d_dtype != HFRK_F16 && d_dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
+    if (rms) {
+        // the prologue exists in the row-split kernel: row-major weights, up to 8 rows, k = 4096 or 8192 (every thread of a
+        // workgroup owns one or two 16-byte pieces of each row)
+        if (packed || m > kRowsRmsMaxM || (k != 4096 && k != 8192) || sa_stride != 0) return HFRK_BAD_SHAPE;
+        if (!rms->input || !rms->residual || !rms->residual_out || !rms->weight || !rms->act_scale) return HFRK_BAD_SHAPE;
+        if (rms->residual_out == rms->residual || rms->residual_out == rms->input) return HFRK_BAD_SHAPE;  // every workgroup reads both
+        if (rms->dtype != HFRK_F16 && rms->dtype != HFRK_BF16) return HFRK_BAD_DTYPE;
+        if ((reinterpret_cast<uintptr_t>(rms->input) | reinterpret_cast<uintptr_t>(rms->residual) |
+             reinterpret_cast<uintptr_t>(rms->residual_out) | reinterpret_cast<uintptr_t>(rms->weight)) & 15)
+            return HFRK_BAD_ALIGNMENT;
+        A = B;  // not read; keeps the checks below on one path
+    }
     if (!A || !B || !D || !scale_a) return HFRK_BAD_SHAPE;
     if ((sa_stride != 0 && sa_stride != 1) || (sb_stride != 0 && sb_stride != 1)) return HFRK_BAD_SHAPE;
     if (epilogue != HFRK_EPILOGUE_NONE && epilogue != HFRK_EPILOGUE_SWIGLU) return HFRK_INVALID_CONFIG;
@@ -945,6 +967,13 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     if (user_plan) {
         p = *user_plan;
         const int rc = check_plan(m, swiglu ? n / 2 : n, k, swiglu, &p, packed);
+        if (rc != HFRK_SUCCESS) return rc;
+        if (rms && (p.wn != -2 || p.wk != (swiglu ? 2 : 1) || p.grid <= m)) return HFRK_INVALID_CONFIG;
+    } else if (rms) {
+        // the row-split plan of the shape, one matrix tile per chunk (SwiGLU: the gate and the up tile)
+        const int n_eff = swiglu ? n / 2 : n;
+        if (make_rows_plan(m, n_eff, k, &p) != HFRK_SUCCESS || p.grid <= m) return HFRK_BAD_SHAPE;
+        const int rc = fill_rows_plan(m, n_eff, k, swiglu ? 2 : 1, p.grid, &p);
         if (rc != HFRK_SUCCESS) return rc;
     } else {
         int rc;
@@ -994,7 +1023,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         HFRK_HIP_TRY(hipGetLastError());
     }
 
-    GemmArgs args;
+    GemmArgs args{};
     args.A = static_cast<const uint8_t*>(A);
     args.B = static_cast<const uint8_t*>(B);
     args.D = D;
@@ -1031,7 +1060,17 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         geometry(args.rows_q + 1, &args.tiles_a, &args.base_a, &args.extra_a);
         geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
         args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)p.slabs - 1) / (uint64_t)p.slabs);
-        return launch_rows_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
+        if (rms) {
+            args.rms_input = static_cast<const uint16_t*>(rms->input);
+            args.rms_residual = static_cast<const uint16_t*>(rms->residual);
+            args.rms_residual_out = static_cast<uint16_t*>(rms->residual_out);
+            args.rms_weight = static_cast<const uint16_t*>(rms->weight);
+            args.rms_act_scale = rms->act_scale;
+            args.rms_epsilon = rms->epsilon;
+            args.rms_dtype = rms->dtype;
+            return launch_rows_kernel(args, p.ch, p.wk, swiglu, true, rows_rms_lds_bytes(p.ch, p.wk, k), stream);
+        }
+        return launch_rows_kernel(args, p.ch, p.wk, swiglu, false, p.lds_bytes, stream);
     }
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, swiglu, p.lds_bytes, stream);
@@ -1180,6 +1219,15 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
                            int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
     return hfrk::gemm_launch(A, B, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, m, n, k, b_stride, d_dtype,
                              epilogue, plan, static_cast<hipStream_t>(stream));
+}
+
+int hfrk_skinny_gemm_rms_fused(const void* input, const void* residual, void* residual_out, const void* rms_weight,
+                               float epsilon, const float* act_scale, int io_dtype, const void* B, void* D, const void* base,
+                               const float* scale_a, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
+                               int k, int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
+    const hfrk::RmsPrologue rms{input, residual, residual_out, rms_weight, act_scale, epsilon, io_dtype};
+    return hfrk::gemm_launch(nullptr, B, D, base, scale_a, 0, scale_b, sb_stride, out_scale, m, n, k, b_stride, d_dtype, epilogue,
+                             plan, static_cast<hipStream_t>(stream), false, false, &rms);
 }
 
 int hfrk_skinny_gemm_packed(const void* A, const void* B_packed, void* D, const void* base, const float* scale_a,

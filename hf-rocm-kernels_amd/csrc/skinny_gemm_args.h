@@ -33,6 +33,15 @@ struct GemmArgs {
     int rows_q, rows_r;
     int tiles_a, base_a, extra_a, tiles_b, base_b, extra_b;
     uint32_t kc_magic;       // ceil(2^32 / slabs): i / slabs == umulhi(i, kc_magic) for the chunk indices of a band
+    // row-split kernel with the RMSNorm prologue (A is then unused): residual_out <- input + residual,
+    // activations = e4m3fn(rmsnorm(residual_out) * weight / act_scale[0]), built in every workgroup's LDS
+    const uint16_t* rms_input;
+    const uint16_t* rms_residual;
+    uint16_t* rms_residual_out;
+    const uint16_t* rms_weight;
+    const float* rms_act_scale;
+    float rms_epsilon;
+    int rms_dtype;           // HFRK_F16 / HFRK_BF16 of input, residual and weight
     float* ws;               // fp32 partial sums that cross workgroups
     uint32_t ws_bytes;       // size of ws: accesses beyond it are dropped by the buffer range check
     int* counters;           // arrival counters, zero between launches
@@ -57,7 +66,14 @@ constexpr bool stream_variant_exists(int act_loads, int row_tiles, bool swiglu =
 // act_loads = ceil(m/4), row_tiles = 16-row matrix tiles per chunk (1 or 2).  Needs k >= 512.
 // swiglu: gate rows [0, n/2), up rows [n/2, n); row_tiles must be 2 (a gate and an up tile per chunk), bands and tiles count
 // the n/2 output columns, D is fp8 [m, n/2]
-int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream);
+// rms: the RMSNorm prologue (args.rms_*): up to 8 rows (act_loads <= 2), k = 4096 or 8192, row_tiles 1 (plain epilogue) or 2 (swiglu);
+// lds_bytes is then rows_rms_lds_bytes(act_loads, row_tiles, k)
+int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, bool rms, int lds_bytes, hipStream_t stream);
+constexpr int kRowsRmsMaxM = 8;
+constexpr int kRowsRmsRedBytes = 8 * kGemmWaves * 4;  // per-row, per-wave partial sums of squares
+constexpr int rows_rms_lds_bytes(int act_loads, int row_tiles, int k) {
+    return kGemmWaves * row_tiles * kTileBytes + kRowsRmsRedBytes + 4 * act_loads * k;  // weight tiles, partial sums, [4*act_loads, k] fp8
+}
 constexpr int kRowsMaxM = 16;
 constexpr int rows_lds_bytes(int row_tiles) { return kGemmWaves * (row_tiles + 1) * kTileBytes; }
 constexpr bool rows_variant_exists(int act_loads, int row_tiles) {

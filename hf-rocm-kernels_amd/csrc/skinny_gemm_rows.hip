@@ -43,11 +43,21 @@ __device__ __forceinline__ uint32_t pack16(float lo, float hi, bool bf16) {
 // output columns (n/2 of them); a chunk pairs up to 16 gate rows with the up rows of the same columns (RT = 2: the gate
 // tile and the up tile), and the epilogue stores e4m3fn(silu(gate) * up / out_scale) into D [m, n/2] instead of the two
 // 16-bit projections -- the SwiGLU kernel of csrc/op_src/swiglu/swiglu_vectorized.cu:27-97 as the GEMM's epilogue.
-template <int MA, int RT, bool SWIGLU>
+// RMS: the residual RMSNorm that feeds the projection runs as the kernel's prologue (the reference launches it as a
+// kernel of its own, hf_rocm_kernels/combined_ops/llama_mlp.py:23-33, csrc/op_src/residual_rms/residual_rms_vectorized.cu:13-172).
+// Every workgroup adds input and residual, reduces the sums of squares of all rows and writes the normalised, quantised
+// rows [4*MA, k] into its own LDS, in the order the matrix cores read them; the loop then takes the activation operands
+// from there and loads nothing but weights.  Thread t owns the 16-byte pieces t and t + 512 of every row, the partial
+// sums are added in the stand-alone kernel's order, and both use the same per-piece functions: the activations are
+// bit-identical to residual_rms's.  Workgroup r stores row r of the summed residual (to a buffer of its own: every
+// workgroup reads the old residual, so it cannot be updated in place).  k = 4096 or 8192, up to 8 rows.
+template <int MA, int RT, bool SWIGLU, bool RMS>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const GemmArgs a) {
     static_assert(!SWIGLU || RT == 2, "the SwiGLU epilogue pairs one gate tile with one up tile");
+    static_assert(!RMS || MA <= 2, "the RMSNorm prologue keeps every row in registers: up to 8 rows");
     constexpr uint32_t kOutOfRange = 0x80000000u;
-    constexpr int kWaveLds = (RT + 1) * kTileBytes;  // RT weight tiles, one activation tile
+    constexpr int kWaveLds = (RMS ? RT : RT + 1) * kTileBytes;  // RT weight tiles, one activation tile (RMS: rows staged once instead)
+    constexpr int R = 4 * MA;                                  // activation rows the MA loads (or the staged block) hold
     constexpr int kSlotStride = kWaveLds / 16;       // in v4f
 
     extern __shared__ __align__(16) uint8_t lds[];
@@ -87,9 +97,11 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     uint32_t irow_off = (uint32_t)irow0 * (uint32_t)a.b_stride;
     auto issue_chunk = [&]() __attribute__((always_inline)) {
         const uint32_t kbyte = (uint32_t)ikc * 256u;
+        if constexpr (!RMS) {
 #pragma unroll
-        for (int t = 0; t < MA; ++t)
-            aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+            for (int t = 0; t < MA; ++t)
+                aq[t] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_lane_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.k), 0, 0);
+        }
 #pragma unroll
         for (int t = 0; t < 4 * RT; ++t) {  // unit t of the tile; a unit the tile does not have reads as zero, without traffic
             // SWIGLU: loads 0..3 fetch the tile's gate rows, loads 4..7 the up rows of the same columns, n/2 rows further down
@@ -130,6 +142,85 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
 
     uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its activation tile
     uint8_t* const ta = tw + RT * kTileBytes;
+    // RMS: behind all weight tiles the partial sums of squares [R][8 waves], then the staged rows.  16-byte piece p of row r
+    // (p = kc*16 + h*8 + lg*2 + half: K chunk, 128-byte half, lane group, low / high 16 bytes of the lane's 32) lies at
+    // ((((kc*2 + h)*2 + half)*4 + lg)*R + r)*16: what the lanes (lg, li < R) of one operand read fetch is contiguous.
+    // Rows from m on are neither computed nor staged: what the matrix cores read there feeds output rows nobody stores.
+    float* const red = reinterpret_cast<float*>(lds + kGemmWaves * kWaveLds);
+    uint8_t* const stage = lds + kGemmWaves * kWaveLds + kRowsRmsRedBytes;
+    if constexpr (RMS) {
+        const bool rbf16 = a.rms_dtype == HFRK_BF16;
+        const uint32_t row_bytes = (uint32_t)a.k * 2u;
+        const __amdgpu_buffer_rsrc_t in_rsrc = make_rsrc(a.rms_input, (uint32_t)a.m * row_bytes);
+        const __amdgpu_buffer_rsrc_t res_rsrc = make_rsrc(a.rms_residual, (uint32_t)a.m * row_bytes);
+        const __amdgpu_buffer_rsrc_t out_rsrc = make_rsrc(a.rms_residual_out, (uint32_t)a.m * row_bytes);
+        const __amdgpu_buffer_rsrc_t nw_rsrc = make_rsrc(a.rms_weight, row_bytes);
+        const bool two = a.k > 4096;  // pieces t and t + 512 of a row (k = 8192), else piece t only
+        uint4 z[R][2], wreg[2];
+        float ssq[R];
+#pragma unroll
+        for (int it = 0; it < 2; ++it)
+            wreg[it] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(nw_rsrc, (it == 0 || two) ? (tid + it * kGemmThreads) * 16 : (int)kOutOfRange, 0, 0));
+        // every row is requested before the first is used: one memory latency for the block, not one per row (the stores
+        // of the summed residual below would otherwise keep the next row's loads behind them)
+        uint4 xin[R][2], xres[R][2];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (r >= a.m) continue;  // uniform
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const int off = (it == 0 || two) ? (int)((uint32_t)r * row_bytes + (uint32_t)(tid + it * kGemmThreads) * 16u) : (int)kOutOfRange;
+                xin[r][it] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, off, 0, 0));
+                xres[r][it] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(res_rsrc, off, 0, 0));
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            ssq[r] = 0.f;
+            if (r >= a.m) continue;
+#pragma unroll
+            for (int it = 0; it < 2; ++it)
+                z[r][it] = rbf16 ? rms_add_square<HFRK_BF16>(xin[r][it], xres[r][it], ssq[r]) : rms_add_square<HFRK_F16>(xin[r][it], xres[r][it], ssq[r]);
+        }
+        if (g < a.m) {  // workgroup g stores row g of the summed residual
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (r != g) continue;
+#pragma unroll
+                for (int it = 0; it < 2; ++it) {
+                    const int off = (it == 0 || two) ? (int)((uint32_t)r * row_bytes + (uint32_t)(tid + it * kGemmThreads) * 16u) : (int)kOutOfRange;
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, z[r][it]), out_rsrc, off, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (r >= a.m) continue;
+            const float s = wave_sum(ssq[r]);
+            if (lane == 0) red[r * kGemmWaves + wv] = s;
+        }
+        __syncthreads();
+        const float inv_scale = 1.f / a.rms_act_scale[0];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (r >= a.m) continue;
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < kGemmWaves; ++w) total += red[r * kGemmWaves + w];
+            const float norm = rsqrtf(total / (float)a.k + a.rms_epsilon);
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                if (it == 1 && !two) break;
+                const uint2 q = rbf16 ? rms_scale_to_fp8<HFRK_BF16>(z[r][it], wreg[it], norm, inv_scale)
+                                      : rms_scale_to_fp8<HFRK_F16>(z[r][it], wreg[it], norm, inv_scale);
+                const int v = tid + it * kGemmThreads;  // 8 K-bytes v*8 .. v*8+8: half of 16-byte piece p = v / 2
+                const int p = v >> 1;
+                const int chunk = p >> 4, h = (p >> 3) & 1, grp = (p >> 1) & 3, half = p & 1;
+                *reinterpret_cast<uint2*>(stage + ((((chunk * 2 + h) * 2 + half) * 4 + grp) * R + r) * 16 + (v & 1) * 8) = q;
+            }
+        }
+        __syncthreads();
+    }
     int wr_off[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -252,8 +343,10 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
 #pragma unroll
     for (int u = 0; u < RT; ++u) acc[u] = part_h[u] = v4f{0.f, 0.f, 0.f, 0.f};
     for (int i = 0; i < count; ++i) {
+        if constexpr (!RMS) {
 #pragma unroll
-        for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
+            for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
+        }
 #pragma unroll
         for (int t = 0; t < 4 * RT; ++t) *reinterpret_cast<v4i*>(tw + (t / 4) * kTileBytes + wr_off[t % 4]) = wq[t];
         pre_cur = pre_next;
@@ -276,8 +369,16 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
                 const v4i hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
                 wop[h][rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
-            const v4i lo = *reinterpret_cast<const v4i*>(ta + rd_off[h]);
-            const v4i hi = *reinterpret_cast<const v4i*>(ta + (rd_off[h] ^ 16));
+            v4i lo, hi;
+            if constexpr (RMS) {
+                // lanes li >= R read row R - 1 again: they feed output rows that are never stored
+                const uint8_t* const piece = stage + ((((kc * 2 + h) * 2) * 4 + lg) * R + min(li, R - 1)) * 16;
+                lo = *reinterpret_cast<const v4i*>(piece);
+                hi = *reinterpret_cast<const v4i*>(piece + 4 * R * 16);
+            } else {
+                lo = *reinterpret_cast<const v4i*>(ta + rd_off[h]);
+                hi = *reinterpret_cast<const v4i*>(ta + (rd_off[h] ^ 16));
+            }
             aop[h] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the requests above ahead of the MFMAs below
@@ -332,9 +433,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     epilogue(row0_l, units_l, acc, pre_l);
 }
 
-template <int MA, int RT, bool SWIGLU>
+template <int MA, int RT, bool SWIGLU, bool RMS>
 static int launch_rows_one(const GemmArgs& args, int lds_bytes, hipStream_t stream) {
-    auto kern = skinny_gemm_rows_kernel<MA, RT, SWIGLU>;
+    auto kern = skinny_gemm_rows_kernel<MA, RT, SWIGLU, RMS>;
     static bool attr_done[kMaxDevices] = {};
     int dev = 0;
     HFRK_HIP_TRY(hipGetDevice(&dev));
@@ -347,14 +448,21 @@ static int launch_rows_one(const GemmArgs& args, int lds_bytes, hipStream_t stre
     return HFRK_SUCCESS;
 }
 
-int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream) {
-    if (!rows_variant_exists(act_loads, row_tiles) || lds_bytes != rows_lds_bytes(row_tiles)) return HFRK_INVALID_CONFIG;
+int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, bool rms, int lds_bytes, hipStream_t stream) {
+    if (!rows_variant_exists(act_loads, row_tiles)) return HFRK_INVALID_CONFIG;
     if (swiglu && row_tiles != 2) return HFRK_INVALID_CONFIG;
+    if (rms) {  // variants: up to 8 rows; one tile per chunk with the plain epilogue, gate + up tile with SwiGLU
+        if (act_loads > 2 || row_tiles != (swiglu ? 2 : 1) || (args.k != 4096 && args.k != 8192)) return HFRK_INVALID_CONFIG;
+        if (lds_bytes != rows_rms_lds_bytes(act_loads, row_tiles, args.k)) return HFRK_INVALID_CONFIG;
+        if (act_loads == 1) return swiglu ? launch_rows_one<1, 2, true, true>(args, lds_bytes, stream) : launch_rows_one<1, 1, false, true>(args, lds_bytes, stream);
+        return swiglu ? launch_rows_one<2, 2, true, true>(args, lds_bytes, stream) : launch_rows_one<2, 1, false, true>(args, lds_bytes, stream);
+    }
+    if (lds_bytes != rows_lds_bytes(row_tiles)) return HFRK_INVALID_CONFIG;
 #define HFRK_ROWS_CASE(MA_)                                                                     \
     case MA_:                                                                                   \
-        if (swiglu) return launch_rows_one<MA_, 2, true>(args, lds_bytes, stream);              \
-        return row_tiles == 1 ? launch_rows_one<MA_, 1, false>(args, lds_bytes, stream)         \
-                              : launch_rows_one<MA_, 2, false>(args, lds_bytes, stream);
+        if (swiglu) return launch_rows_one<MA_, 2, true, false>(args, lds_bytes, stream);       \
+        return row_tiles == 1 ? launch_rows_one<MA_, 1, false, false>(args, lds_bytes, stream)  \
+                              : launch_rows_one<MA_, 2, false, false>(args, lds_bytes, stream);
     switch (act_loads) {
         HFRK_ROWS_CASE(1)
         HFRK_ROWS_CASE(2)

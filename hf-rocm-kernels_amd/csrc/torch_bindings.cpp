@@ -340,6 +340,67 @@ int64_t skinny_gemm_fused(at::Tensor& A, at::Tensor& B, at::Tensor& D, const std
     return gemm_fused_common(A, B, false, B.size(1), D, base, scale_a, scale_b, out_scale, epilogue, intermediate_dtype);
 }
 
+// skinny_gemm_fused with the residual RMSNorm of its activations as the kernel's prologue (no reference counterpart as one
+// op: the reference launches residual_rms, then skinny_gemm).  residual_out <- input + residual; the GEMM multiplies
+// e4m3fn(rmsnorm(residual_out) * rms_weight / act_scale) by B.  Returns the launcher's status: 7 (HFRK_BAD_SHAPE) where the
+// prologue does not exist (more than 8 rows, k other than 4096 / 8192, rows that do not deal out evenly).
+int64_t skinny_gemm_rms_fused(at::Tensor& input, at::Tensor& residual, at::Tensor& residual_out, at::Tensor& rms_weight,
+                              double epsilon, at::Tensor& act_scale, at::Tensor& B, at::Tensor& D,
+                              const std::optional<at::Tensor>& base, at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b,
+                              const std::optional<at::Tensor>& out_scale, int64_t epilogue, int64_t intermediate_dtype) {
+    TORCH_CHECK(input.dim() == 2 && input.is_contiguous(), "input must be a contiguous [m, k] tensor");
+    const int io = dtype16(input, "input");
+    const int64_t m = input.size(0), k = input.size(1);
+    TORCH_CHECK(residual.sizes() == input.sizes() && residual.is_contiguous() && residual.scalar_type() == input.scalar_type(),
+                "residual must be a contiguous tensor with input's shape and dtype");
+    TORCH_CHECK(residual_out.sizes() == input.sizes() && residual_out.is_contiguous() && residual_out.scalar_type() == input.scalar_type(),
+                "residual_out must be a contiguous tensor with input's shape and dtype");
+    TORCH_CHECK(rms_weight.dim() == 1 && rms_weight.size(0) == k && rms_weight.is_contiguous() && rms_weight.scalar_type() == input.scalar_type(),
+                "rms_weight must be a contiguous [k] tensor of input's dtype");
+    TORCH_CHECK(act_scale.numel() == 1 && act_scale.scalar_type() == at::kFloat, "act_scale must be one float32");
+    TORCH_CHECK(scale_a.numel() == 1 && scale_a.scalar_type() == at::kFloat, "scale_a must be one float32");
+    check_fp8(B, "B");
+    TORCH_CHECK(B.dim() == 2 && B.size(0) == k && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
+    const int64_t n = B.size(1);
+    for (const at::Tensor* t : {&residual, &residual_out, &rms_weight, &act_scale, &B, &D, &scale_a}) check_same_device(input, *t, "every tensor");
+    const float* scale_b_ptr = nullptr;
+    int sb_stride = 0;
+    if (scale_b.has_value()) {
+        TORCH_CHECK(scale_b->scalar_type() == at::kFloat && scale_b->is_contiguous() && (scale_b->numel() == 1 || scale_b->numel() == n),
+                    "scale_b must be float32 with 1 or n elements");
+        check_same_device(input, *scale_b, "scale_b");
+        scale_b_ptr = scale_b->data_ptr<float>();
+        sb_stride = scale_b->numel() == 1 ? 0 : 1;
+    }
+    int d_dtype;
+    const void* base_ptr = nullptr;
+    const float* out_scale_ptr = nullptr;
+    if (epilogue == HFRK_EPILOGUE_SWIGLU) {
+        TORCH_CHECK(n % 2 == 0 && D.dim() == 2 && D.size(0) == m && D.size(1) == n / 2 && D.is_contiguous(), "D must be a contiguous [m, n/2] tensor");
+        check_fp8(D, "D");
+        TORCH_CHECK(out_scale.has_value() && out_scale->numel() == 1 && out_scale->scalar_type() == at::kFloat, "out_scale must be one float32");
+        check_same_device(input, *out_scale, "out_scale");
+        TORCH_CHECK(!base.has_value(), "base cannot be combined with the SwiGLU epilogue");
+        TORCH_CHECK(intermediate_dtype == HFRK_F16 || intermediate_dtype == HFRK_BF16, "intermediate_dtype must be 0 (float16) or 1 (bfloat16)");
+        d_dtype = (int)intermediate_dtype;
+        out_scale_ptr = out_scale->data_ptr<float>();
+    } else {
+        TORCH_CHECK(D.dim() == 2 && D.size(0) == m && D.size(1) == n && D.is_contiguous(), "D must be a contiguous [m, n] tensor");
+        d_dtype = dtype16(D, "D");
+        if (base.has_value()) {
+            TORCH_CHECK(base->sizes() == D.sizes() && base->is_contiguous() && base->scalar_type() == D.scalar_type(),
+                        "base must be a contiguous tensor with D's shape and dtype");
+            check_same_device(input, *base, "base");
+            base_ptr = base->data_ptr();
+        }
+    }
+    DeviceScope scope(input);
+    return hfrk_skinny_gemm_rms_fused(input.data_ptr(), residual.data_ptr(), residual_out.data_ptr(), rms_weight.data_ptr(), (float)epsilon,
+                                      act_scale.data_ptr<float>(), io, B.data_ptr(), D.data_ptr(), base_ptr, scale_a.data_ptr<float>(),
+                                      scale_b_ptr, sb_stride, out_scale_ptr, (int)m, (int)n, (int)k, (int)B.stride(1), d_dtype,
+                                      (int)epilogue, nullptr, current_stream(input));
+}
+
 // The same on a weight in the load format of hfrk_pack_weight (no reference counterpart).
 int64_t skinny_gemm_packed(at::Tensor& A, at::Tensor& B_packed, int64_t n, at::Tensor& D, const std::optional<at::Tensor>& base,
                            at::Tensor& scale_a, const std::optional<at::Tensor>& scale_b, const std::optional<at::Tensor>& out_scale,
@@ -438,6 +499,11 @@ TORCH_LIBRARY(_HFRK_C, ops) {
         "skinny_gemm_fused(Tensor A, Tensor B, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "
         "Tensor? out_scale, int epilogue, int intermediate_dtype) -> int");
     ops.impl("skinny_gemm_fused", c10::kCUDA, &skinny_gemm_fused);
+    ops.def(
+        "skinny_gemm_rms_fused(Tensor input, Tensor residual, Tensor! residual_out, Tensor rms_weight, float epsilon, "
+        "Tensor act_scale, Tensor B, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, Tensor? out_scale, "
+        "int epilogue, int intermediate_dtype) -> int");
+    ops.impl("skinny_gemm_rms_fused", c10::kCUDA, &skinny_gemm_rms_fused);
 
     ops.def(
         "skinny_gemm_packed(Tensor A, Tensor B_packed, int n, Tensor! D, Tensor? base, Tensor scale_a, Tensor? scale_b, "

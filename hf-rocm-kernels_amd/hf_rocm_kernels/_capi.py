@@ -72,6 +72,7 @@ SIGNATURES = {
     "hfrk_skinny_gemm_ex": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_noalloc": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
+    "hfrk_skinny_gemm_rms_fused": (_i, [_p, _p, _p, _p, _f, _p, _i, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_packed_weight_bytes": (ctypes.c_size_t, [_i, _i]),
     "hfrk_pack_weight": (_i, [_p, _i, _i, _p, _i, _i, _p]),
     "hfrk_unpack_weight": (_i, [_p, _p, _i, _i, _i, _p]),

@@ -16,7 +16,7 @@ import hf_rocm_kernels._HFRK_C  # noqa: F401  (registers torch.ops._HFRK_C)
 
 _RETURNS_NOTHING = ("increment", "residual_rms", "swiglu", "pack_weight", "pack_weight_scaled", "unpack_weight", "reencode_fnuz",
                     "residual_rms_dynamic", "swiglu_dynamic", "quantize_fp8", "skinny_gemm_checked")
-_RETURNS_STATUS = ("skinny_gemm_tb", "skinny_gemm_scaled", "skinny_gemm_fused", "skinny_gemm_packed")
+_RETURNS_STATUS = ("skinny_gemm_tb", "skinny_gemm_scaled", "skinny_gemm_fused", "skinny_gemm_packed", "skinny_gemm_rms_fused")
 
 
 def _nothing(*args, **kwargs) -> None:

@@ -3,7 +3,7 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor
 
-from hf_rocm_kernels import residual_rms, skinny_gemm, skinny_gemm_add, skinny_gemm_scaled, skinny_gemm_swiglu, swiglu
+from hf_rocm_kernels import residual_rms, skinny_gemm, skinny_gemm_add, skinny_gemm_rms, skinny_gemm_scaled, skinny_gemm_swiglu, swiglu
 
 
 def llama_mlp_combined_ops(
@@ -21,6 +21,7 @@ def llama_mlp_combined_ops(
     down_gemm_hp: Tuple[Optional[int], Optional[int]] = (None, None),
     add_residual: bool = False,
     fused: bool = False,
+    rms_prologue: bool = False,
 ) -> Tuple[Tensor, Tensor]:
     """Decoder MLP sub-block as four launches on one stream (reference: combined_ops/llama_mlp.py:7-60):
     residual RMSNorm -> fp8, gate_up GEMM, SwiGLU -> fp8, down GEMM.
@@ -37,9 +38,25 @@ def llama_mlp_combined_ops(
       nothing is zeroed beforehand (the GEMMs overwrite), and with add_residual the down projection reads the
       residual as its addend instead of accumulating onto a copy.  Same arithmetic, same roundings.
 
+    - rms_prologue (with fused): two launches where the library has the prologue (up to 8 rows, hidden 4096 or 8192,
+      row-major gate_up weight): the RMSNorm runs inside the gate_up GEMM, in every workgroup.  Same bits as the three
+      launches, but the summed residual is returned as a new tensor and `residual` is left as it was (every workgroup of
+      the fused launch reads the old residual, so it cannot be updated in place).
+
     RMSNorm and SwiGLU zero the buffer the following GEMM accumulates into, as in the reference.
     Returns (mlp_output, residual)."""
     del gate_up_gemm_hp, down_gemm_hp
+    if fused and rms_prologue:
+        swiglu_out, residual = skinny_gemm_rms(attn_output, residual, rms_weight, rms_epsilon, gate_up_input_scale, gate_up_weight,
+                                               gate_up_output_scale, None, None, out_scale=down_input_scale)
+        if add_residual:
+            mlp_output = skinny_gemm_add(swiglu_out, down_weight, down_output_scale, None, base=residual)
+        else:
+            mlp_output = torch.empty(size=(attn_output.size(0), down_weight.size(1)), dtype=attn_output.dtype,
+                                     device=attn_output.device)
+            skinny_gemm_scaled(swiglu_out, down_weight, down_output_scale,
+                               torch.ones(1, device=attn_output.device), output=mlp_output)
+        return mlp_output, residual
     if fused:
         normalized, residual = residual_rms(input=attn_output, residual=residual, weight=rms_weight, epsilon=rms_epsilon,
                                             scale_tensor=gate_up_input_scale)

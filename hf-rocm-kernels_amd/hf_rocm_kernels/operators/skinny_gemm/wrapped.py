@@ -245,3 +245,70 @@ def skinny_gemm_swiglu(
     _fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU,
            _capi.BF16 if intermediate_dtype == torch.bfloat16 else _capi.F16)
     return output
+
+
+def rms_prologue_available(m: int, n_rows: int, k: int, b) -> bool:
+    """Whether `skinny_gemm_rms` runs as one launch: the RMSNorm prologue exists in the row-split kernel -- row-major
+    weights, up to 8 rows, k = 4096 or 8192, and weight rows (output columns with SwiGLU) that deal out evenly over the
+    workgroups, which the library's planner decides (`hfrk_skinny_gemm_plan` returns a row-split plan, wn = -2)."""
+    if isinstance(b, PackedWeight) or m > 8 or k not in (4096, 8192) or torch.compiler.is_compiling():
+        return False
+    try:
+        return _capi.plan(m, n_rows, k).wn == -2
+    except RuntimeError:
+        return False
+
+
+def skinny_gemm_rms(
+    input: Tensor,
+    residual: Tensor,
+    rms_weight: Tensor,
+    epsilon: float,
+    act_scale: Tensor,
+    b: Tensor,
+    scale: Tensor,
+    scale_b: Optional[Tensor] = None,
+    base: Optional[Tensor] = None,
+    out_scale: Optional[Tensor] = None,
+    output: Optional[Tensor] = None,
+    residual_out: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor]:
+    """Residual RMSNorm and the projection that consumes it, in one launch where the prologue exists
+    (`rms_prologue_available`), else as `residual_rms` followed by the GEMM -- same bits either way:
+        residual_out = input + residual                                  (16-bit add)
+        a            = float8_e4m3fn(rmsnorm(residual_out) * rms_weight / act_scale)
+        output       = base + scale * scale_b * (a @ b)                  (out_scale None), or
+        output       = float8_e4m3fn(silu(gate) * up / out_scale)        (out_scale given: b is a gate_up weight)
+    `scale` is one float32 (activation scale x weight scale), `scale_b` optionally one per output channel.
+    Unlike `residual_rms`, which updates `residual` in place, the sum goes to `residual_out` (allocated if None; it
+    must not alias `input` or `residual`): every workgroup of the fused launch reads the old residual.
+    Returns (output, residual_out).  No counterpart in the reference, which launches the two kernels
+    (combined_ops/llama_mlp.py:23-41)."""
+    m, k = input.shape
+    n = b.size(1)
+    swiglu = out_scale is not None
+    dtype = input.dtype
+    if output is None:
+        output = torch.empty((m, n // 2), dtype=torch.float8_e4m3fn, device=input.device) if swiglu else \
+            torch.empty((m, n), dtype=dtype, device=input.device)
+    if not rms_prologue_available(m, n // 2 if swiglu else n, k, b):
+        from ..residual_rms import residual_rms
+        res = residual.clone() if residual_out is None else residual_out.copy_(residual)
+        normalized, res = residual_rms(input=input, residual=res, weight=rms_weight, epsilon=epsilon, scale_tensor=act_scale)
+        if swiglu:
+            skinny_gemm_swiglu(normalized, b, scale, scale_b, out_scale, output=output, intermediate_dtype=dtype)
+        elif base is not None:
+            skinny_gemm_add(normalized, b, scale, scale_b, base, output=output)
+        else:
+            skinny_gemm_scaled(normalized, b, scale, scale_b if scale_b is not None else torch.ones(1, device=input.device), output=output)
+        return output, res
+    if residual_out is None:
+        residual_out = torch.empty_like(residual)
+    assert residual_out.data_ptr() not in (input.data_ptr(), residual.data_ptr()), "residual_out must not alias input or residual"
+    assert scale.numel() == 1 and scale.dtype == torch.float32, "Expected scale to be one float32"
+    status = torch.ops._HFRK_C.skinny_gemm_rms_fused(
+        input, residual, residual_out, rms_weight, float(epsilon), act_scale, b, output, base, scale.reshape(-1),
+        None if scale_b is None else scale_b.contiguous().view(-1), out_scale,
+        _capi.EPILOGUE_SWIGLU if swiglu else _capi.EPILOGUE_NONE, _capi.BF16 if dtype == torch.bfloat16 else _capi.F16)
+    _raise_on_status(status, "skinny_gemm_rms_fused")
+    return output, residual_out

@@ -202,6 +202,22 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
                            const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k,
                            int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
 
+/* hfrk_skinny_gemm_fused with the residual RMSNorm that feeds it as the kernel's prologue: one launch for what the
+ * reference's chain runs as `residual_rms` followed by `skinny_gemm` (hf_rocm_kernels/combined_ops/llama_mlp.py:23-41;
+ * csrc/op_src/residual_rms/residual_rms_dispatch.cu:8-63 for the norm).
+ *   residual_out <- input + residual (one 16-bit add; a buffer of its own: every workgroup reads the old residual);
+ *   A = e4m3fn(rmsnorm(residual_out) * rms_weight / act_scale[0]) is built in every workgroup's LDS, bit-identical to what
+ *   hfrk_residual_rms writes; then the GEMM and its epilogue as in hfrk_skinny_gemm_fused, with scale_a one float
+ *   (activation scale x weight scale).  input, residual, residual_out [m,k] and rms_weight [k] are io_dtype (f16/bf16),
+ *   16-byte aligned.
+ * Exists in the row-split kernel: row-major weights, m <= 8, k = 4096 or 8192, a shape whose rows deal out evenly over the
+ * workgroups (HFRK_BAD_SHAPE otherwise: callers then run the two launches); an explicit plan must be a row-split plan with
+ * wk = 1 (2 with the SwiGLU epilogue). */
+int hfrk_skinny_gemm_rms_fused(const void* input, const void* residual, void* residual_out, const void* rms_weight,
+                               float epsilon, const float* act_scale, int io_dtype, const void* B, void* D, const void* base,
+                               const float* scale_a, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
+                               int k, int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
+
 /* Weight load format (no reference counterpart: the reference streams row-major weights through an LDS ring,
  * csrc/op_src/skinny_gemm/producers/n_full_tiles.cu:4-127, and stores fn bits viewed as fnuz,
  * hf_rocm_kernels/utils/fp8.py:27-29).  A weight packed once when the model is loaded is read by the GEMM as one
