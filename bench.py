@@ -1,6 +1,6 @@
 """Headline benchmark: FP8 skinny GEMM on Llama decode linear shapes, one MI355X.
 
-Default workload (`--workload llama3-8b`, BASELINE's second configuration): a step is one pass over
+Default workload (`--workload llama3-8b`, the headline configuration): a step is one pass over
 M in {1, 2, 4, 8, 16} x the four projection shapes qkv (6144, 4096), o_proj (4096, 4096), gate_up (28672, 4096),
 down (4096, 14336) -- 20 calls of `hf_rocm_kernels.skinny_gemm` (FP8 e4m3fn activations and weights, per-tensor
 scales, bf16 output accumulated into a zeroed buffer, as the reference's callers do).  All inputs are resident in
@@ -582,7 +582,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--ms", type=str, default=None,
                     help="comma-separated activation row counts replacing the workload's own (e.g. 32,64 for the MLP block above 16 rows); "
-                         "the result then describes that variant of the workload, not BASELINE's")
+                         "the result then describes that variant of the workload, not the named one")
     ap.add_argument("--packed", action="store_true",
                     help="weights in the library's packed load format (hfrk_pack_weight) instead of row-major [N, K]")
     ap.add_argument("--cpu-budget", type=float, default=20.0)

@@ -223,7 +223,7 @@ def test_per_token_and_per_channel_scales(m, n, k):
 
 
 def test_full_size_properties_llama70b_down():
-    """BASELINE's largest K (8192 x 28672), checked through size-independent properties instead of the oracle:
+    """The largest K of the Llama-3-70B shapes (8192 x 28672), checked through size-independent properties instead of the oracle:
     zero activations give the bias back bit for bit, a one-hot activation row returns a scaled weight column
     exactly, and the product is linear in the output scale."""
     from hf_rocm_kernels import skinny_gemm
@@ -572,7 +572,7 @@ def test_every_shipped_plan_table_entry_computes_what_the_planner_s_plan_compute
     assert float(want.float().abs().mean()) > 0.1
 
 
-# ---- BASELINE config 3 (Llama-3-70B, unsharded) at full size against the oracle ------------------------------------------
+# ---- the Llama-3-70B projections (unsharded) at full size against the oracle ------------------------------------------
 
 def _check_columns_against_oracle(cases, b_codes_nk, sw, cols=4096):
     """cases: [(label, out [m,n] on the device, a [m,k] fp8 on the host, sa [1 or m] on the host)].  The oracle's two
@@ -607,7 +607,7 @@ def _check_columns_against_oracle(cases, b_codes_nk, sw, cols=4096):
 @pytest.mark.parametrize("name,n,k", [("qkv", 10240, 8192), ("o_proj", 8192, 8192), ("gate_up", 57344, 8192),
                                       ("down", 8192, 28672)])
 def test_llama3_70b_shapes_match_the_oracle(name, n, k):
-    """Every (N, K) of BASELINE's Llama-3-70B configuration, row-major at M = 1, 8, 32 and from the packed weight at
+    """Every (N, K) of the Llama-3-70B projections, row-major at M = 1, 8, 32 and from the packed weight at
     M = 8, through the operator (so with the plan the installed table or the planner gives the shape), against the
     exact oracle at full size."""
     from hf_rocm_kernels import plan_table, skinny_gemm, skinny_gemm_scaled

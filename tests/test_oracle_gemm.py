@@ -95,7 +95,7 @@ def test_fp32_reference_within_one_ulp_of_exact(per_token, per_channel):
 
 
 def test_config1_shape_matches_torch_scaled_mm_on_cpu():
-    """BASELINE config 1 (M=8, N=K=4096, per-tensor amax/448 scales): torch's own CPU _scaled_mm on e4m3fn -- the
+    """The reference test shape (M=8, N=K=4096, per-tensor amax/448 scales): torch's own CPU _scaled_mm on e4m3fn -- the
     library routine behind the reference's oracle -- agrees with the restated path to one bf16 ulp."""
     m, n, k = 8, 4096, 4096
     g = torch.Generator().manual_seed(0)

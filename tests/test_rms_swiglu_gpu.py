@@ -132,7 +132,7 @@ def test_rms_rejects_bad_epsilon_and_mixed_dtypes():
 @pytest.mark.parametrize("add_residual", [False, True])
 @pytest.mark.parametrize("m", [1, 8, 16])
 def test_llama_mlp_chain(m, add_residual, fused):
-    """BASELINE config 4: hidden 4096, gate_up 28672x4096, down 4096x14336, eps 1e-5, weight ~ 1+N(0,0.1), bf16."""
+    """The Llama-3-8B MLP block: hidden 4096, gate_up 28672x4096, down 4096x14336, eps 1e-5, weight ~ 1+N(0,0.1), bf16."""
     from hf_rocm_kernels.combined_ops.llama_mlp import llama_mlp_combined_ops
     from hf_rocm_kernels.utils.fp8 import amax_scale, fp8_quantize
     from oracle import llama_mlp as omlp
@@ -174,7 +174,7 @@ def test_llama_mlp_chain(m, add_residual, fused):
 @pytest.mark.parametrize("add_residual", [False, True])
 @pytest.mark.parametrize("m", [1, 8, 16])
 def test_llama_mlp_chain_stage_by_stage(m, add_residual, fused):
-    """BASELINE config 4 held to the strict bar, one stage at a time: every stage of the device chain is compared with the
+    """The Llama-3-8B MLP block held to the strict bar, one stage at a time: every stage of the device chain is compared with the
     oracle's next stage fed with the device's own output of the stage before (so that an fp8 boundary flip upstream cannot
     move the comparison), and the block's result must be, bit for bit, what these stages give when run one by one.
     Order of the chain: hf_rocm_kernels/combined_ops/llama_mlp.py:23-59 of the reference."""
