@@ -291,9 +291,9 @@ def skinny_gemm_rms(
     if output is None:
         output = torch.empty((m, n // 2), dtype=torch.float8_e4m3fn, device=input.device) if swiglu else \
             torch.empty((m, n), dtype=dtype, device=input.device)
-    if not rms_prologue_available(m, n // 2 if swiglu else n, k, b):
+    def two_launches(res: Tensor) -> Tuple[Tensor, Tensor]:
         from ..residual_rms import residual_rms
-        res = residual.clone() if residual_out is None else residual_out.copy_(residual)
+        res.copy_(residual)
         normalized, res = residual_rms(input=input, residual=res, weight=rms_weight, epsilon=epsilon, scale_tensor=act_scale)
         if swiglu:
             skinny_gemm_swiglu(normalized, b, scale, scale_b, out_scale, output=output, intermediate_dtype=dtype)
@@ -302,13 +302,18 @@ def skinny_gemm_rms(
         else:
             skinny_gemm_scaled(normalized, b, scale, scale_b if scale_b is not None else torch.ones(1, device=input.device), output=output)
         return output, res
+
     if residual_out is None:
         residual_out = torch.empty_like(residual)
     assert residual_out.data_ptr() not in (input.data_ptr(), residual.data_ptr()), "residual_out must not alias input or residual"
+    if not rms_prologue_available(m, n // 2 if swiglu else n, k, b):
+        return two_launches(residual_out)
     assert scale.numel() == 1 and scale.dtype == torch.float32, "Expected scale to be one float32"
     status = torch.ops._HFRK_C.skinny_gemm_rms_fused(
         input, residual, residual_out, rms_weight, float(epsilon), act_scale, b, output, base, scale.reshape(-1),
         None if scale_b is None else scale_b.contiguous().view(-1), out_scale,
         _capi.EPILOGUE_SWIGLU if swiglu else _capi.EPILOGUE_NONE, _capi.BF16 if dtype == torch.bfloat16 else _capi.F16)
+    if status == _capi.BAD_SHAPE:  # the library has no prologue for this shape after all (its own planner decides)
+        return two_launches(residual_out)
     _raise_on_status(status, "skinny_gemm_rms_fused")
     return output, residual_out
