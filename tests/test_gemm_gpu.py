@@ -106,7 +106,8 @@ def test_default_plan_matches_oracle(m, n, k):
 @pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
                                    (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024),
                                    (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096),
-                                   (32, 1040, 8192), (48, 4096, 4096), (9, 528, 16384)])
+                                   (32, 1040, 8192), (48, 4096, 4096), (9, 528, 16384),
+                                   (5, 1027, 768), (16, 4099, 512), (2, 2050, 1024), (11, 1533, 2048)])   # n % 4 != 0: element-wise stores
 def test_every_plan_gives_the_same_answer(m, n, k):
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=7)
