@@ -25,7 +25,7 @@ def _inputs(m, n, k, dtype, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,n,k", [(1, 6144, 4096), (4, 4096, 4096), (8, 28672, 4096), (3, 10240, 8192), (8, 8192, 8192), (5, 3584, 4096)])
+@pytest.mark.parametrize("m,n,k", [(1, 6144, 4096), (4, 4096, 4096), (8, 28672, 4096), (3, 10240, 8192), (8, 8192, 8192), (5, 3584, 4096), (4, 4098, 4096)])
 def test_plain_projection_with_the_norm_as_prologue(m, n, k, dtype):
     from hf_rocm_kernels import residual_rms, skinny_gemm_add, skinny_gemm_rms, skinny_gemm_scaled
     from hf_rocm_kernels.operators.skinny_gemm import rms_prologue_available
