@@ -1060,6 +1060,14 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         geometry(args.rows_q + 1, &args.tiles_a, &args.base_a, &args.extra_a);
         geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
         args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)p.slabs - 1) / (uint64_t)p.slabs);
+        {
+            // chunks per wave in the band height most workgroups have
+            const int tiles = 2 * args.rows_r > p.grid ? args.tiles_a : args.tiles_b;
+            const long run8 = (long)tiles * p.slabs;  // eight waves' worth
+            const bool same_offset = run8 % 8 == 0 && (run8 / 8) % 16 == 0;
+            const bool shared_lines = p.ch >= 3 && p.panels >= 4 * p.grid;  // (bands of 2-3 units lose 3 %: 2304 x 16384)
+            args.k_rotate = (b_stride % 4096 == 0 && (same_offset || shared_lines)) ? 1 : 0;
+        }
         if (rms) {
             args.rms_input = static_cast<const uint16_t*>(rms->input);
             args.rms_residual = static_cast<const uint16_t*>(rms->residual);

@@ -33,6 +33,12 @@ struct GemmArgs {
     int rows_q, rows_r;
     int tiles_a, base_a, extra_a, tiles_b, base_b, extra_b;
     uint32_t kc_magic;       // ceil(2^32 / slabs): i / slabs == umulhi(i, kc_magic) for the chunk indices of a band
+    // row-split kernel: workgroup g walks k from chunk g mod slabs on (and wraps round).  Set for rows a multiple of 4 KB
+    // apart when the 2048 waves of a launch would otherwise ask for the same offset within 4 KB at every moment: either
+    // because every wave's run of chunks is a multiple of 16 long (13312 x 16384 at 8 rows: 41.7 us without, 33.7 with;
+    // 16384 x 16384: 53.4 / 43.5), or because from 9 activation rows on all workgroups pull the same activation lines out
+    // of L2 together (6144 x 4096 at 16 rows: 7.10 / 6.77; bands of at least 4 units).  Elsewhere the rotation costs 1-3 %.
+    int k_rotate;
     // row-split kernel with the RMSNorm prologue (A is then unused): residual_out <- input + residual,
     // activations = e4m3fn(rmsnorm(residual_out) * weight / act_scale[0]), built in every workgroup's LDS
     const uint16_t* rms_input;

@@ -92,6 +92,11 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     const uint32_t a_lane_off = (uint32_t)lg * (uint32_t)a.k + (uint32_t)li * 16u;
     v4i wq[4 * RT], aq[MA];
     int itile = tile, ikc = kc;                                        // chunk being requested
+    // Where the host asks for it, the point in k at which a workgroup starts is rotated by its index: chunk kc of a tile
+    // reads K bytes ((kc + g) mod KC) * 256.  Every tile still sums all of k once, but the 2048 waves of a launch, which
+    // advance in step, no longer ask for the same offset within their rows at the same moment (see k_rotate).
+    const int rot = a.k_rotate ? g - (int)__umulhi((uint32_t)g, a.kc_magic) * KC : 0;  // g mod KC
+    int ikr = kc + rot - (kc + rot >= KC ? KC : 0);                    // its rotated position in k
     int iunits = ubase + (itile < uextra ? 1 : 0);                     // its tile's height in units
     int irow0 = 4 * (u0 + itile * ubase + min(itile, uextra));        // its tile's first row
     uint32_t irow_off = (uint32_t)irow0 * (uint32_t)a.b_stride;
@@ -100,7 +105,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     // instructions themselves stand there (about 30 instructions fewer per chunk; 0.2-0.4 us on a 10-20 us launch).
     uint32_t a_voff[MA], w_voff[4 * RT];
     auto chunk_offsets = [&]() __attribute__((always_inline)) {
-        const uint32_t kbyte = (uint32_t)ikc * 256u;
+        const uint32_t kbyte = (uint32_t)ikr * 256u;
 #pragma unroll
         for (int t = 0; t < MA; ++t) a_voff[t] = a_lane_off + kbyte + (uint32_t)(4 * t) * (uint32_t)a.k;
 #pragma unroll
@@ -121,6 +126,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
         for (int t = 0; t < 4 * RT; ++t) wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)w_voff[t], 0, 2 /* nt */);
     };
     auto next_chunk = [&]() __attribute__((always_inline)) {
+        if (++ikr == KC) ikr = 0;
         if (++ikc == KC) {
             ikc = 0;
             irow0 += 4 * iunits;
@@ -346,6 +352,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     const Pre pre_l = prefetch(row0_l, units_l, finisher);
 
     // ---- streaming loop ---------------------------------------------------------------------------------------------
+    int kr = ikr;                                            // rotated k position of the chunk being multiplied
     int units = iunits;                                      // geometry of the tile being multiplied
     int row0 = 4 * (u0 + tile * ubase + min(tile, uextra));
     Pre pre_next = prefetch(row0, units, count > 0 && kc == KC - 1 && !(kb0 != 0)), pre_cur;
@@ -389,7 +396,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
             v4i lo, hi;
             if constexpr (RMS) {
                 // lanes li >= R read row R - 1 again: they feed output rows that are never stored
-                const uint8_t* const piece = stage + ((((kc * 2 + h) * 2) * 4 + lg) * R + min(li, R - 1)) * 16;
+                const uint8_t* const piece = stage + ((((kr * 2 + h) * 2) * 4 + lg) * R + min(li, R - 1)) * 16;
                 lo = *reinterpret_cast<const v4i*>(piece);
                 hi = *reinterpret_cast<const v4i*>(piece + 4 * R * 16);
             } else {
@@ -406,6 +413,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
                 acc[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h][rt], aop[h], acc[rt], 0, 0, 0, 0, 0, 0);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        if constexpr (RMS) {
+            if (++kr == KC) kr = 0;
+        }
         if (++kc == KC) {  // a tile ends inside this wave's run
             if (tile == tile_h && kb0 != 0) {  // its first chunks belong to an earlier wave
 #pragma unroll

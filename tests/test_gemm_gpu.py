@@ -122,6 +122,34 @@ def test_every_plan_gives_the_same_answer(m, n, k):
             raise AssertionError(f"plan {p.as_dict()}: {e}")
 
 
+@pytest.mark.parametrize("m,n,k,grid,rt", [(3, 2048, 4096, 4, 1), (8, 2048, 4096, 2, 2), (5, 1024, 8192, 2, 1), (1, 4096, 4096, 8, 1),
+                                          (16, 2048, 4096, 4, 2), (12, 1024, 8192, 3, 1), (9, 6144, 4096, 256, 2)])
+def test_row_split_plans_that_rotate_k(m, n, k, grid, rt):
+    """Row-split plans under which every workgroup starts at its own point in k and wraps round (rows a multiple of 4 KB
+    apart and either every wave's run a multiple of 16 chunks long, or 9+ activation rows on bands of 4+ units): against
+    the oracle, on a contiguous weight and on one whose rows are 8 KB / 12 KB apart with NaN codes behind k (a rotation that
+    left the row's k bytes could not pass), plain and accumulating."""
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    units = (n + 3) // 4
+    per_band = units // grid
+    tiles = -(-per_band // (4 * rt))
+    assert (tiles * (k // 256)) % 128 == 0 or (m >= 9 and units >= 4 * grid), "the case is meant to switch the rotation on"
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k + grid, per_token=True, per_channel=True)
+    wide = torch.full((n, k + 4096), 0x7F, dtype=torch.uint8, device="cuda")
+    wide[:, :k] = b.t().contiguous().view(torch.uint8)
+    b_view = wide.view(torch.float8_e4m3fn)[:, :k].t()
+    plan = _capi.GemmPlan(1, -2, rt, (m + 3) // 4, grid, units, k // 256, 8 * (rt + 1) * 4096)
+    for weight in (b, b_view):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        run_ex(a, weight, sa, sw, out, accumulate=False, plan=plan)
+        check_against_oracle(out, a, b, sa, sw)
+    base = torch.randn(m, n, generator=torch.Generator().manual_seed(3)).to(torch.float16).cuda()
+    out = base.clone()
+    run_ex(a, b_view, sa, sw, out, accumulate=True, plan=plan)
+    check_against_oracle(out, a, b, sa, sw, base=base)
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096 + 128), (8, 1000, 640), (16, 6144, 4096 + 64), (32, 2048, 1152),
                                    (33, 1024, 640), (64, 4096, 4096 + 128), (5, 256, 144), (3, 128, 16), (12, 4096, 1008)])
 def test_k_that_ends_inside_a_chunk(m, n, k):

@@ -62,6 +62,33 @@ def test_gate_up_projection_with_norm_prologue_and_swiglu_epilogue(m, n, k, dtyp
     assert got.view(torch.uint8).any()
 
 
+@pytest.mark.parametrize("m,n,k,grid", [(3, 2048, 4096, 4), (7, 1024, 8192, 8), (2, 4096, 4096, 8)])
+def test_prologue_under_a_plan_that_rotates_k(m, n, k, grid):
+    """Explicit row-split plans whose workgroups start at different points in k (every wave's run is a multiple of 16
+    chunks): the staged activations are then read from the rotated position too.  Same bits as the two launches under
+    the same plan."""
+    from hf_rocm_kernels import _capi, residual_rms
+    lib = _capi.load()
+    x, res, w_norm, w8, act_scale, scale = _inputs(m, n, k, torch.bfloat16, seed=m + n + grid)
+    units = n // 4
+    assert (-(-(units // grid) // 4) * (k // 256)) % 128 == 0
+    plan = _capi.GemmPlan(1, -2, 1, (m + 3) // 4, grid, units, k // 256, 8 * 2 * 4096)
+    one = torch.ones(1).cuda()
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16).cuda()
+    res_out = torch.empty_like(res)
+    assert lib.hfrk_skinny_gemm_rms_fused(x.data_ptr(), res.data_ptr(), res_out.data_ptr(), w_norm.data_ptr(), 1e-5, act_scale.data_ptr(),
+                                          _capi.BF16, w8.data_ptr(), out.data_ptr(), None, scale.data_ptr(), None, 0, None, m, n, k, k,
+                                          _capi.BF16, _capi.EPILOGUE_NONE, ctypes.byref(plan), None) == _capi.SUCCESS
+    torch.cuda.synchronize()
+    normalized, want_res = residual_rms(x, res.clone(), w_norm, 1e-5, scale_tensor=act_scale)
+    want = torch.empty_like(out)
+    assert lib.hfrk_skinny_gemm_ex(normalized.data_ptr(), w8.data_ptr(), want.data_ptr(), scale.data_ptr(), 0, one.data_ptr(), 0, m, n, k, k,
+                                   _capi.BF16, 0, ctypes.byref(plan), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(res_out, want_res) and torch.equal(out, want)
+    assert not out.isnan().any() and out.float().abs().sum() > 0
+
+
 @pytest.mark.parametrize("add_residual", [False, True])
 @pytest.mark.parametrize("m", [1, 4, 8])
 def test_mlp_block_in_two_launches_equals_the_three_launch_block(m, add_residual):
