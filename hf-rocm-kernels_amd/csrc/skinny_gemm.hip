@@ -621,7 +621,7 @@ static int make_stream_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 // m <= 16: every workgroup owns a band of weight rows (4-row units dealt out evenly) and all of k (skinny_gemm_rows.hip).
 // plan: wn = -2, wk = matrix tiles per chunk, ch = activation loads, panels = 4-row units, slabs = k / 256.
 static int fill_rows_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk_gemm_plan* plan) {
-    const int act_loads = (m + 3) / 4;
+    const int act_loads = rows_act_loads(m);
     if (m > kRowsMaxM || !rows_variant_exists(act_loads, row_tiles) || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
     const long units = (n + 3) / 4;
     long grid = grid_hint > 0 ? grid_hint : kNumCU;
@@ -634,7 +634,7 @@ static int fill_rows_plan(int m, int n, int k, int row_tiles, int grid_hint, hfr
     plan->grid = (int)grid;
     plan->panels = (int)units;
     plan->slabs = k / 256;
-    plan->lds_bytes = rows_lds_bytes(row_tiles);
+    plan->lds_bytes = rows_lds_bytes(row_tiles, act_loads);
     return HFRK_SUCCESS;
 }
 
@@ -664,7 +664,7 @@ static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         else if (m <= 4 && 4 * busiest <= 48 && units >= 4 * kNumCU) grid = 2 * kNumCU;  // bands of at least 8 rows
     }
     const long rows_per_band = 4 * ((units + grid - 1) / grid);
-    const int row_tiles = (m >= 9 && rows_per_band >= 24) ? 2 : 1;
+    const int row_tiles = (m > 16 || (m >= 9 && rows_per_band >= 24)) ? 2 : 1;
     return fill_rows_plan(m, n, k, row_tiles, (int)grid, plan);
 }
 
@@ -707,6 +707,7 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 //   m <= 16          row-split kernel (a band of weight rows and all of k per workgroup) when the rows deal out evenly,
 //                    else the wave-stream kernel (chunk runs that may split a tile's k between workgroups); K-split kernel
 //                    for weights of at most 2048 chunks (8 MB) when one window of it covers k
+//   17 <= m <= 32    row-split kernel with two activation tiles on bands of 24-64 rows and moderate k (rule below)
 //   m  > 16          K-split kernel (activations in registers) when one window of it covers k; otherwise the
 //                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
 //                    4 row waves x 2 K waves almost everywhere; 2 x 4 for narrow weights (n <= 2048: more K parallelism
@@ -754,6 +755,17 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
         if (!packed && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // (row-major weights only)
         return make_stream_plan(m, n, k, plan);
     }
+    // 17..32 rows in the row-split kernel (two activation tiles): every workgroup then pulls all m x k activation bytes out
+    // of L2 itself, which pays while a band's chunks stay large against them and k is moderate.  Measured against the
+    // kernels below at 24 / 32 rows: 6144 x 4096 7.96 / 8.70 us against 9.54 / 9.55 (K-split, 1.5 tiles per workgroup),
+    // 8192 x 8192 13.5 / 14.3 against 15.2 / 15.2, 10240 x 8192 18.5 against 19.4 at 24, 13312 x 16384 38.2 against 41.0 at
+    // 24, 16384 x 2048 8.9 against 10.3; slower on bands of 16 rows (4096 x 14336 +2 / +12 %), on k = 28672 (+3 / +7 %) and
+    // on the largest weights at 32 rows (57344 x 8192 +9 %).
+    if (m <= kRowsMaxM && !packed) {
+        const long band_rows = 4 * (((long)(n + 3) / 4 + kNumCU - 1) / kNumCU);
+        const bool fits = m <= 24 ? (band_rows >= 24 && band_rows <= 64 && k <= 16384) : (band_rows >= 24 && band_rows <= 32 && k <= 8192);
+        if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
+    }
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     const double weight_mb = (double)n * k / 1.0e6;
     int first = 4;
@@ -771,12 +783,12 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
     if (swiglu && p->wn != 0 && p->wn != -2 && p->wn != -1) return HFRK_INVALID_CONFIG;  // the workgroup kernel has no fused epilogue
     if (p->wn == -2) {  // row-split decomposition: wk = matrix tiles per chunk, ch = activation loads
         if (packed) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
-        if (swiglu && p->wk != 2) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows
+        if (swiglu && (p->wk != 2 || p->ch > 4)) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows; up to 16 rows
         if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
         if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
         if (p->m_tiles != 1 || p->panels != (n + 3) / 4 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
         if (p->grid < 1 || p->grid > kMaxGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
-        if (p->lds_bytes != rows_lds_bytes(p->wk)) return HFRK_INVALID_CONFIG;
+        if (p->lds_bytes != rows_lds_bytes(p->wk, p->ch)) return HFRK_INVALID_CONFIG;
         // a band's chunk indices stay far below 2^32 / slabs (the kernel divides by multiplying with a reciprocal)
         if (((long)p->panels / p->grid / 4 + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;
         return HFRK_SUCCESS;

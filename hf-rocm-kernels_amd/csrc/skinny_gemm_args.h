@@ -80,10 +80,11 @@ constexpr int kRowsRmsRedBytes = 8 * kGemmWaves * 4;  // per-row, per-wave parti
 constexpr int rows_rms_lds_bytes(int act_loads, int row_tiles, int k) {
     return kGemmWaves * row_tiles * kTileBytes + kRowsRmsRedBytes + 4 * act_loads * k;  // weight tiles, partial sums, [4*act_loads, k] fp8
 }
-constexpr int kRowsMaxM = 16;
-constexpr int rows_lds_bytes(int row_tiles) { return kGemmWaves * (row_tiles + 1) * kTileBytes; }
+constexpr int kRowsMaxM = 32;  // 17..32 rows: act_loads 6 (up to 24 rows) or 8, two matrix tiles per chunk, plain epilogue
+constexpr int rows_act_loads(int m) { return m <= 16 ? (m + 3) / 4 : m <= 24 ? 6 : 8; }
+constexpr int rows_lds_bytes(int row_tiles, int act_loads) { return kGemmWaves * (row_tiles + (act_loads + 3) / 4) * kTileBytes; }
 constexpr bool rows_variant_exists(int act_loads, int row_tiles) {
-    return act_loads >= 1 && act_loads <= 4 && (row_tiles == 1 || row_tiles == 2);
+    return (act_loads >= 1 && act_loads <= 4 && (row_tiles == 1 || row_tiles == 2)) || ((act_loads == 6 || act_loads == 8) && row_tiles == 2);
 }
 
 // K-split kernel (skinny_gemm_ksplit.hip): the 8 waves of a workgroup split a K window of 8*wave_k bytes

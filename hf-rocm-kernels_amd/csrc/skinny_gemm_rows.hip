@@ -55,13 +55,15 @@ template <int MA, int RT, bool SWIGLU, bool RMS>
 __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const GemmArgs a) {
     static_assert(!SWIGLU || RT == 2, "the SwiGLU epilogue pairs one gate tile with one up tile");
     static_assert(!RMS || MA <= 2, "the RMSNorm prologue keeps every row in registers: up to 8 rows");
+    constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles: 2 from 17 rows on (plain epilogue, two matrix tiles per chunk)
+    static_assert(MT == 1 || (MT == 2 && RT == 2 && !SWIGLU && !RMS), "above 16 rows: two weight tiles per chunk, plain epilogue");
     constexpr uint32_t kOutOfRange = 0x80000000u;
-    constexpr int kWaveLds = (RMS ? RT : RT + 1) * kTileBytes;  // RT weight tiles, one activation tile (RMS: rows staged once instead)
+    constexpr int kWaveLds = (RMS ? RT : RT + MT) * kTileBytes;  // RT weight tiles, MT activation tiles (RMS: rows staged once instead)
     constexpr int R = 4 * MA;                                  // activation rows the MA loads (or the staged block) hold
     constexpr int kSlotStride = kWaveLds / 16;       // in v4f
 
     extern __shared__ __align__(16) uint8_t lds[];
-    // A wave's partial sums (RT x 64 lanes x 16 bytes) go to the start of its own weight tiles, which are dead by then.
+    // A wave's partial sums (MT x RT x 64 lanes x 16 bytes) go to the start of its own weight tiles, which are dead by then.
     v4f* const slots = reinterpret_cast<v4f*>(lds);
 
     const int tid = threadIdx.x;
@@ -148,15 +150,19 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     const bool vec = SWIGLU || (a.n & 3) == 0;  // then a lane's four outputs are all inside n and aligned
     const bool per_channel = a.scale_b && a.sb_stride;
     const bool bf16 = a.d_dtype == HFRK_BF16;
-    // lane li holds the accumulator column of activation row li
-    const float sa = a.scale_a[(long)min(li, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+    // lane li holds the accumulator column of activation row 16 mt + li
+    float sa_mt[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+        sa_mt[mt] = a.scale_a[(long)min(16 * mt + li, a.m - 1) * a.sa_stride] * ((a.scale_b && !a.sb_stride) ? a.scale_b[0] : 1.0f);
+    const float sa = sa_mt[0];
     float inv_out_scale = 1.0f;
     if constexpr (SWIGLU) {
         const float os = a.out_scale[0];
         inv_out_scale = os != 0.f ? 1.0f / os : 1.0f;
     }
 
-    uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its activation tile
+    uint8_t* const tw = lds + wv * kWaveLds;  // this wave's RT weight tiles, then its activation tile(s)
     uint8_t* const ta = tw + RT * kTileBytes;
     // RMS: behind all weight tiles the partial sums of squares [R][8 waves], then the staged rows.  16-byte piece p of row r
     // (p = kc*16 + h*8 + lg*2 + half: K chunk, 128-byte half, lane group, low / high 16 bytes of the lane's 32) lies at
@@ -249,15 +255,14 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
 
     // Old D values (accumulate mode) and per-channel scales of a tile whose first row is `row0` (aligned n only; ragged
     // n fetches in the epilogue).  Nothing is requested when nothing is wanted.
-    struct Pre { v2i d[RT]; v4i sb[RT]; };
+    struct Pre { v2i d[MT * RT]; v4i sb[RT]; };
     const bool want_pre = vec && (accumulate || per_channel);
     auto prefetch = [&](int row0, int units, bool wanted) __attribute__((always_inline)) {
         Pre p;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            p.sb[rt] = v4i{0, 0, 0, 0};
-            p.d[rt] = v2i{0, 0};
-        }
+        for (int rt = 0; rt < RT; ++rt) p.sb[rt] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < MT * RT; ++u) p.d[u] = v2i{0, 0};
         if (wanted && want_pre) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -265,14 +270,16 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
                 const int n0 = row0 + 4 * ul + (SWIGLU ? rt * (a.n >> 1) : 0);  // its first weight row (= scale channel)
                 const bool ok = ul < units && n0 < a.n;
                 p.sb[rt] = __builtin_amdgcn_raw_buffer_load_b128(sb_rsrc, (per_channel && ok) ? n0 * 4 : (int)kOutOfRange, 0, 0);
-                p.d[rt] = __builtin_amdgcn_raw_buffer_load_b64(base_rsrc, (accumulate && ok && li < a.m) ? (int)(((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    p.d[mt * RT + rt] = __builtin_amdgcn_raw_buffer_load_b64(base_rsrc, (accumulate && ok && 16 * mt + li < a.m) ? (int)(((uint32_t)(16 * mt + li) * (uint32_t)a.n + (uint32_t)n0) * 2u) : (int)kOutOfRange, 0, 0);
             }
         }
         return p;
     };
 
     // scale, add D (accumulate mode), round once, store: lane holds D[li][n0 + v], v = 0..3, n0 = row0 + 16*rt + 4*lg
-    auto epilogue = [&](int row0, int units, const v4f (&acc)[RT], const Pre& pre) __attribute__((always_inline)) {
+    auto epilogue = [&](int row0, int units, const v4f (&acc)[MT * RT], const Pre& pre) __attribute__((always_inline)) {
         if constexpr (SWIGLU) {
             // acc[0] = gate, acc[1] = up of output columns n0 .. n0+3.  The unfused chain stores both projections in the
             // 16-bit dtype between its two kernels: round them the same way before the activation.
@@ -294,17 +301,20 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
             return;
         }
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
+        for (int u = 0; u < MT * RT; ++u) {
+            const int mt = u / RT, rt = u % RT;
+            const int arow = 16 * mt + li;  // activation row = row of D
+            const float sa = sa_mt[mt];
             const int ul = 4 * rt + lg;
             const int n0 = row0 + 4 * ul;
-            const bool live = li < a.m && ul < units && n0 < a.n;
-            const uint32_t d_off = ((uint32_t)li * (uint32_t)a.n + (uint32_t)n0) * 2u;
+            const bool live = arow < a.m && ul < units && n0 < a.n;
+            const uint32_t d_off = ((uint32_t)arow * (uint32_t)a.n + (uint32_t)n0) * 2u;
             if (vec) {
                 const v4f sb = __builtin_bit_cast(v4f, pre.sb[rt]);
-                const uint32_t d0 = (uint32_t)pre.d[rt][0], d1 = (uint32_t)pre.d[rt][1];
+                const uint32_t d0 = (uint32_t)pre.d[u][0], d1 = (uint32_t)pre.d[u][1];
                 float r[4];
 #pragma unroll
-                for (int v = 0; v < 4; ++v) r[v] = acc[rt][v] * (per_channel ? sa * sb[v] : sa);
+                for (int v = 0; v < 4; ++v) r[v] = acc[u][v] * (per_channel ? sa * sb[v] : sa);
                 if (accumulate) {
                     if (bf16) {
                         r[0] += __uint_as_float(d0 << 16); r[1] += __uint_as_float(d0 & 0xffff0000u);
@@ -323,7 +333,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
                     const uint32_t off = (live && n0 + v < a.n) ? d_off + 2u * v : kOutOfRange;
                     const uint32_t old = accumulate ? (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(base_rsrc, (int)off, 0, 0) : 0u;
                     const float sbv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(sb_rsrc, (live && per_channel && n0 + v < a.n) ? (n0 + v) * 4 : (int)kOutOfRange, 0, 0));
-                    float r = acc[rt][v] * (per_channel ? sa * sbv : sa);
+                    float r = acc[u][v] * (per_channel ? sa * sbv : sa);
                     if (accumulate) r += bf16 ? bf16_bits_to_float((uint16_t)old) : f16_bits_to_float((uint16_t)old);
                     __builtin_amdgcn_raw_buffer_store_b16((short)(pack16(r, 0.f, bf16) & 0xffffu), d_rsrc, (int)off, 0, 0);
                 }
@@ -356,9 +366,9 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     int units = iunits;                                      // geometry of the tile being multiplied
     int row0 = 4 * (u0 + tile * ubase + min(tile, uextra));
     Pre pre_next = prefetch(row0, units, count > 0 && kc == KC - 1 && !(kb0 != 0)), pre_cur;
-    v4f acc[RT], part_h[RT];
+    v4f acc[MT * RT], part_h[MT * RT];  // [activation tile][weight tile]
 #pragma unroll
-    for (int u = 0; u < RT; ++u) acc[u] = part_h[u] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < MT * RT; ++u) acc[u] = part_h[u] = v4f{0.f, 0.f, 0.f, 0.f};
     if (count > 1) {  // the second chunk's offsets
         next_chunk();
         chunk_offsets();
@@ -366,7 +376,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     for (int i = 0; i < count; ++i) {
         if constexpr (!RMS) {
 #pragma unroll
-            for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + wr_off[t]) = aq[t];
+            for (int t = 0; t < MA; ++t) *reinterpret_cast<v4i*>(ta + (t / 4) * kTileBytes + wr_off[t % 4]) = aq[t];
         }
 #pragma unroll
         for (int t = 0; t < 4 * RT; ++t) *reinterpret_cast<v4i*>(tw + (t / 4) * kTileBytes + wr_off[t % 4]) = wq[t];
@@ -384,7 +394,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // every operand of the chunk is requested from LDS before the first MFMA
-        v8i wop[2][RT], aop[2];
+        v8i wop[2][RT], aop[2][MT];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -393,6 +403,8 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
                 const v4i hi = *reinterpret_cast<const v4i*>(tw + rt * kTileBytes + (rd_off[h] ^ 16));
                 wop[h][rt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
             v4i lo, hi;
             if constexpr (RMS) {
                 // lanes li >= R read row R - 1 again: they feed output rows that are never stored
@@ -400,17 +412,18 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
                 lo = *reinterpret_cast<const v4i*>(piece);
                 hi = *reinterpret_cast<const v4i*>(piece + 4 * R * 16);
             } else {
-                lo = *reinterpret_cast<const v4i*>(ta + rd_off[h]);
-                hi = *reinterpret_cast<const v4i*>(ta + (rd_off[h] ^ 16));
+                lo = *reinterpret_cast<const v4i*>(ta + mt * kTileBytes + rd_off[h]);
+                hi = *reinterpret_cast<const v4i*>(ta + mt * kTileBytes + (rd_off[h] ^ 16));
             }
-            aop[h] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            aop[h][mt] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the requests above ahead of the MFMAs below
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-                acc[rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h][rt], aop[h], acc[rt], 0, 0, 0, 0, 0, 0);
+            for (int u = 0; u < MT * RT; ++u)
+                acc[u] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wop[h][u % RT], aop[h][u / RT], acc[u], 0, 0, 0, 0, 0, 0);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         if constexpr (RMS) {
@@ -419,12 +432,12 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
         if (++kc == KC) {  // a tile ends inside this wave's run
             if (tile == tile_h && kb0 != 0) {  // its first chunks belong to an earlier wave
 #pragma unroll
-                for (int u = 0; u < RT; ++u) part_h[u] = acc[u];
+                for (int u = 0; u < MT * RT; ++u) part_h[u] = acc[u];
             } else {
                 epilogue(row0, units, acc, pre_cur);  // all of it was ours
             }
 #pragma unroll
-            for (int u = 0; u < RT; ++u) acc[u] = v4f{0.f, 0.f, 0.f, 0.f};
+            for (int u = 0; u < MT * RT; ++u) acc[u] = v4f{0.f, 0.f, 0.f, 0.f};
             kc = 0;
             row0 += 4 * units;
             ++tile;
@@ -434,28 +447,31 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     // a run that lies inside one tile that began in an earlier wave: everything it has is that tile's partial sum
     if (count > 0 && kc != 0 && tile == tile_h && kb0 != 0) {
 #pragma unroll
-        for (int u = 0; u < RT; ++u) part_h[u] = acc[u];
+        for (int u = 0; u < MT * RT; ++u) part_h[u] = acc[u];
     }
 
     // ---- combine the partial tiles of this workgroup ----------------------------------------------------------------
     // Every wave leaves a partial sum (zeros when it has none to hand over), so that the finishing wave can read all seven
     // slots at once and add each with a factor of one or zero: no select, no branch, exact.
 #pragma unroll
-    for (int u = 0; u < RT; ++u) slots[wv * kSlotStride + u * 64 + lane] = hand_over ? part_h[u] : v4f{0.f, 0.f, 0.f, 0.f};
+    for (int u = 0; u < MT * RT; ++u) slots[wv * kSlotStride + u * 64 + lane] = hand_over ? part_h[u] : v4f{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
     if (!finisher) return;
-    v4f other[kGemmWaves][RT];
 #pragma unroll
-    for (int j = 1; j < kGemmWaves; ++j)
+    for (int mt = 0; mt < MT; ++mt) {  // one activation tile at a time: seven waves' partials of it in registers
+        v4f other[kGemmWaves][RT];
 #pragma unroll
-        for (int u = 0; u < RT; ++u) other[j][u] = slots[j * kSlotStride + u * 64 + lane];
+        for (int j = 1; j < kGemmWaves; ++j)
 #pragma unroll
-    for (int j = 1; j < kGemmWaves; ++j) {
-        const float f = (addmask >> j) & 1u ? 1.0f : 0.0f;
+            for (int u = 0; u < RT; ++u) other[j][u] = slots[j * kSlotStride + (mt * RT + u) * 64 + lane];
 #pragma unroll
-        for (int u = 0; u < RT; ++u)
+        for (int j = 1; j < kGemmWaves; ++j) {
+            const float f = (addmask >> j) & 1u ? 1.0f : 0.0f;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[u][v] = __builtin_fmaf(other[j][u][v], f, acc[u][v]);
+            for (int u = 0; u < RT; ++u)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[mt * RT + u][v] = __builtin_fmaf(other[j][u][v], f, acc[mt * RT + u][v]);
+        }
     }
     epilogue(row0_l, units_l, acc, pre_l);
 }
@@ -484,7 +500,11 @@ int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool 
         if (act_loads == 1) return swiglu ? launch_rows_one<1, 2, true, true>(args, lds_bytes, stream) : launch_rows_one<1, 1, false, true>(args, lds_bytes, stream);
         return swiglu ? launch_rows_one<2, 2, true, true>(args, lds_bytes, stream) : launch_rows_one<2, 1, false, true>(args, lds_bytes, stream);
     }
-    if (lds_bytes != rows_lds_bytes(row_tiles)) return HFRK_INVALID_CONFIG;
+    if (lds_bytes != rows_lds_bytes(row_tiles, act_loads)) return HFRK_INVALID_CONFIG;
+    if (act_loads > 4) {  // 17..32 rows: two activation tiles, two weight tiles per chunk, plain epilogue
+        if (swiglu || row_tiles != 2) return HFRK_INVALID_CONFIG;
+        return act_loads == 6 ? launch_rows_one<6, 2, false, false>(args, lds_bytes, stream) : launch_rows_one<8, 2, false, false>(args, lds_bytes, stream);
+    }
 #define HFRK_ROWS_CASE(MA_)                                                                     \
     case MA_:                                                                                   \
         if (swiglu) return launch_rows_one<MA_, 2, true, false>(args, lds_bytes, stream);       \

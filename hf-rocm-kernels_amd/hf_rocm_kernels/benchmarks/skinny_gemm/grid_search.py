@@ -36,11 +36,12 @@ def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.Gemm
                 for g in grids:
                     plans.append(_capi.GemmPlan((ma + 3) // 4, 0, rt, ma, min(g, groups * kc), groups, kc,
                                                 8 * (rt + (ma + 3) // 4) * 4096))
-    if m <= 16 and k >= 512:  # row-split: a band of weight rows per workgroup, one or two matrix tiles per chunk
+    if m <= 32 and k >= 512:  # row-split: a band of weight rows per workgroup, one or two matrix tiles per chunk (two above 16 rows)
         units = -(-n // 4)
-        for rt in (1, 2):
+        ma = (m + 3) // 4 if m <= 16 else (6 if m <= 24 else 8)
+        for rt in ((1, 2) if m <= 16 else (2,)):
             for g in grids:
-                plans.append(_capi.GemmPlan(1, -2, rt, (m + 3) // 4, min(g, units), units, k // 256, 8 * (rt + 1) * 4096))
+                plans.append(_capi.GemmPlan(1, -2, rt, ma, min(g, units), units, k // 256, 8 * (rt + (ma + 3) // 4) * 4096))
     for wave_k in (256, 512, 1024):  # K-split
         if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
             tiles, windows = -(-n // 16), k // (8 * wave_k)

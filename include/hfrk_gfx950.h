@@ -62,17 +62,19 @@ enum hfrk_weight_format { HFRK_WEIGHT_E4M3FN = 0, HFRK_WEIGHT_E4M3FNUZ = 1 };
  * hfrk_skinny_gemm_ex() by an autotuner (counterpart of the knob table in
  * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:42-102 and benchmarks/skinny_gemm/grid_search.py). */
 typedef struct hfrk_gemm_plan {
-    int m_tiles;   /* ceil(m/16): 16-row activation tiles (wave-stream: 1..2, row-split: 1, others: 1..4) */
+    int m_tiles;   /* ceil(m/16): 16-row activation tiles (wave-stream: 1..2, others: 1..4; row-split: always 1, the kernel takes its tiles from ch) */
     int wn;        /* which decomposition:
-                      -2          row-split (m <= 16, k >= 512): every workgroup owns a band of weight rows and all of k
+                      -2          row-split (m <= 32, k >= 512): every workgroup owns a band of weight rows and all of k
                        0          wave-stream (m <= 32): every wave streams its own run of chunks
                       -1          K-split (k % (2048*wk) == 0): the 8 waves of a workgroup split K, activations in registers
                        1..16      workgroup: a panel is wn 16-row weight tiles; the 8 waves are 8/wk row waves x wk K waves,
                                   each row wave takes wn*wk/8 tiles (1, or 2 with ch = 1) */
-    int wk;        /* workgroup: waves spread over K (1, 2, 4, 8), wn*wk = 8 or 16.  wave-stream, row-split: 16-row weight tiles per chunk (1 or 2).
+    int wk;        /* workgroup: waves spread over K (1, 2, 4, 8), wn*wk = 8 or 16.  wave-stream, row-split: 16-row weight tiles per chunk (1 or 2;
+                      row-split above 16 rows: 2).
                       K-split: bytes of K per wave / 256 (1, 2, or 4 with m_tiles <= 2) */
     int ch;        /* workgroup: 256-byte K chunks each wave streams per slab (1 or 2).
-                      wave-stream, row-split: 16-byte activation loads per lane and chunk, ceil(m/4).  K-split: 0 */
+                      wave-stream, row-split: 16-byte activation loads per lane and chunk, ceil(m/4) (row-split above 16 rows:
+                      6 up to 24 rows, else 8).  K-split: 0 */
     int grid;      /* persistent workgroups launched */
     int panels;    /* workgroup: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n / (16*wk)) row groups.
                       K-split: ceil(n/16) row tiles.  row-split: ceil(n/4) units of 4 rows */

@@ -65,11 +65,12 @@ def all_plans(m, n, k):
             groups = (n + 16 * rt - 1) // (16 * rt)
             for grid in sorted({min(g, groups * kc) for g in (256, 200, 7, 512, 1)}):
                 plans.append(_capi.GemmPlan((ma + 3) // 4, 0, rt, ma, grid, groups, kc, 8 * (rt + (ma + 3) // 4) * 4096))
-    if m <= 16 and k >= 512:  # row-split decomposition: bands of rows per workgroup, cut into tiles of different heights
+    if m <= 32 and k >= 512:  # row-split decomposition: bands of rows per workgroup, cut into tiles of different heights
         units = (n + 3) // 4
-        for rt in (1, 2):
+        ma = (m + 3) // 4 if m <= 16 else (6 if m <= 24 else 8)  # above 16 rows: two activation tiles, two weight tiles per chunk
+        for rt in ((1, 2) if m <= 16 else (2,)):
             for grid in sorted({min(g, units) for g in (256, 200, 7, 512, 1, 77)}):
-                plans.append(_capi.GemmPlan(1, -2, rt, (m + 3) // 4, grid, units, k // 256, 8 * (rt + 1) * 4096))
+                plans.append(_capi.GemmPlan(1, -2, rt, ma, grid, units, k // 256, 8 * (rt + (ma + 3) // 4) * 4096))
     for wave_k in (256, 512, 1024):  # K-split decomposition
         if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
             tiles, windows = (n + 15) // 16, k // (8 * wave_k)
@@ -106,7 +107,7 @@ def test_default_plan_matches_oracle(m, n, k):
 @pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
                                    (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024),
                                    (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096),
-                                   (32, 1040, 8192), (48, 4096, 4096), (9, 528, 16384),
+                                   (32, 1040, 8192), (48, 4096, 4096), (9, 528, 16384), (17, 4096, 14336), (24, 1000, 2048), (29, 4100, 1024),
                                    (5, 1027, 768), (16, 4099, 512), (2, 2050, 1024), (11, 1533, 2048)])   # n % 4 != 0: element-wise stores
 def test_every_plan_gives_the_same_answer(m, n, k):
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
