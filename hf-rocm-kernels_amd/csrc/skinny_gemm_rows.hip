@@ -359,7 +359,13 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
         for (int j = 1; j < kGemmWaves; ++j)
             if (j > wv && ((j * TC) >> 3) < e) addmask |= 1u << j;
     }
-    const Pre pre_l = prefetch(row0_l, units_l, finisher);
+    // The D values and scales of that tile are asked for behind the wave's last weight request, not here: the wait for a
+    // chunk also waits for every load issued since, so a request placed here stands in front of the first chunk's use
+    // (accumulate mode, M = 1 / 8: 4096 x 4096 5.11 / 5.38 -> 4.98 / 5.19 us, 28672 x 4096 20.1 / 20.4 -> 19.6 / 20.0,
+    // 4096 x 14336 11.0 -> 10.85).  With two workgroups per CU it is the other way round (6144 x 4096 on 512 workgroups:
+    // 6.04 -> 6.19), so there the request stays here.
+    const bool late_pre = G <= kNumCU && count > 1;
+    Pre pre_l = prefetch(row0_l, units_l, finisher && !late_pre);
 
     // ---- streaming loop ---------------------------------------------------------------------------------------------
     int kr = ikr;                                            // rotated k position of the chunk being multiplied
@@ -385,6 +391,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
             issue_chunk();
             // the chunk that ends a tile this wave finishes in the loop brings the tile's D along
             pre_next = prefetch(irow0, iunits, ikc == KC - 1 && !(itile == tile_h && kb0 != 0));
+            if (i + 2 == count && finisher && late_pre) pre_l = prefetch(row0_l, units_l, true);
             if (i + 2 < count) {  // and the offsets of the one after it, for the next turn
                 next_chunk();
                 chunk_offsets();
