@@ -77,8 +77,8 @@ WORKLOADS = {
         "text": "llama3-70b decode linears: M in {1,4,8,16,32} x qkv(10240,8192) o_proj(8192,8192) gate_up(57344,8192) "
                 "down(8192,28672); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-70B decode shapes, M=1..32 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_rows_kernel (M<=16; down at M=16: hfrk::skinny_gemm_kernel by plan table), "
-                  "hfrk::skinny_gemm_kernel<2,WN,WK,CH,RT> (M=32)",
+        "kernel": "hfrk::skinny_gemm_rows_kernel (M<=16, and o_proj at M=32), hfrk::skinny_gemm_kernel<2,4,2,1,1> (M=32: gate_up, "
+                  "down), hfrk::skinny_gemm_ksplit_kernel<2,1024> (M=32: qkv, by plan table)",
     },
     "scaled-m": {
         "shapes": [("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)],
