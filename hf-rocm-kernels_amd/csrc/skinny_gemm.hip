@@ -656,15 +656,22 @@ static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     long grid = kNumCU;
     const long busiest = (units + grid - 1) / grid;
     if (units * 10 < busiest * grid * 7) return HFRK_INVALID_CONFIG;
+    // A band of exactly 512 KB (every workgroup's weight bytes, rows a power of two apart) is the one size at which the
+    // workgroups, walking their bands in step, keep landing on the same memory channels even with the start in k rotated:
+    // 0.65 of peak where the neighbouring sizes reach 0.75-0.78 (16384 x 8192, 8192 x 16384, 32768 x 4096: 25.5-25.7 us;
+    // 256 KB, 1 MB and 1.5 MB bands are fine).  Two matrix tiles per chunk walk it differently (22.0-22.7 us), and a grid
+    // that would create such bands is not taken for the sake of whole tiles (14336 x 8192: 22.4 us on 224 workgroups,
+    // 19.4 on 256).
+    auto half_mb_bands = [&](long g) { return units % g == 0 && 4 * (units / g) * (long)k == (1L << 19); };
     if (units % (4 * grid) != 0) {
         long whole = 0;
         for (long g = kNumCU - 8; g >= 7 * kNumCU / 8; g -= 8)
-            if (units % (4 * g) == 0) { whole = g; break; }
+            if (units % (4 * g) == 0 && !half_mb_bands(g)) { whole = g; break; }
         if (whole) grid = whole;
         else if (m <= 4 && 4 * busiest <= 48 && units >= 4 * kNumCU) grid = 2 * kNumCU;  // bands of at least 8 rows
     }
     const long rows_per_band = 4 * ((units + grid - 1) / grid);
-    const int row_tiles = (m > 16 || (m >= 9 && rows_per_band >= 24)) ? 2 : 1;
+    const int row_tiles = (m > 16 || (m >= 9 && rows_per_band >= 24) || (half_mb_bands(grid) && rows_per_band >= 24)) ? 2 : 1;
     return fill_rows_plan(m, n, k, row_tiles, (int)grid, plan);
 }
 
