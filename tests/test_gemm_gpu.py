@@ -104,6 +104,23 @@ def test_default_plan_matches_oracle(m, n, k):
     check_against_oracle(out, a, b, sa, sw)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 16384, 8192), (8, 8192, 16384), (5, 14336, 8192), (24, 8192, 8192), (32, 6144, 4096), (19, 16384, 2048)])
+def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
+    """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224) and the 17..32
+    row variants of the row-split kernel, as the planner chooses them: against the oracle, plain and accumulating."""
+    from hf_rocm_kernels import _capi
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    assert _capi.plan(m, n, k).wn == -2
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k, per_token=True, per_channel=True)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    run_ex(a, b, sa, sw, out, accumulate=False)
+    check_against_oracle(out, a, b, sa, sw)
+    base = torch.randn(m, n, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).cuda()
+    out = base.clone()
+    run_ex(a, b, sa, sw, out, accumulate=True)
+    check_against_oracle(out, a, b, sa, sw, base=base)
+
+
 @pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
                                    (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024),
                                    (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096),

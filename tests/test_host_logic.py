@@ -256,6 +256,30 @@ def test_plans_for_k_that_ends_inside_a_chunk():
     assert lib.hfrk_skinny_gemm_plan(8, 1000, 648, ctypes.byref(p)) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
 
 
+def test_row_split_plans_for_17_to_32_rows_and_for_half_megabyte_bands():
+    """The planner's row-split rules beyond 16 rows and around 512 KB bands: 17..32 rows run the row-split kernel with a
+    second activation tile (ch = 6 up to 24 rows, else 8; two weight tiles per chunk) on bands of 24..64 rows with
+    moderate k; a weight whose bands would come to exactly 512 KB gets two weight tiles per chunk at any row count, and
+    a grid chosen for whole tiles is not taken when it creates such bands."""
+    p = _capi.GemmPlan()
+    lib = _capi.load()
+    plan = lambda m, n, k: (lib.hfrk_skinny_gemm_plan(m, n, k, ctypes.byref(p)), p.wn, p.wk, p.ch, p.grid, p.lds_bytes)
+    assert plan(24, 8192, 8192) == (0, -2, 2, 6, 256, 8 * 4 * 4096)
+    assert plan(32, 8192, 8192) == (0, -2, 2, 8, 256, 8 * 4 * 4096)
+    assert plan(20, 6144, 4096)[1:4] == (-2, 2, 6) and plan(32, 6144, 4096)[1:4] == (-2, 2, 8)
+    assert plan(32, 10240, 8192)[1] != -2      # bands of 40 rows: up to 24 rows only
+    assert plan(24, 4096, 14336)[1] != -2      # bands of 16 rows
+    assert plan(24, 8192, 28672)[1] != -2      # k above 16384
+    assert plan(33, 8192, 8192)[1] != -2
+    # 512 KB bands
+    assert plan(1, 16384, 8192)[1:5] == (-2, 2, 1, 256)
+    assert plan(8, 8192, 16384)[1:5] == (-2, 2, 2, 256)
+    assert plan(4, 32768, 4096)[1:5] == (-2, 2, 1, 256)
+    assert plan(1, 14336, 8192)[1:5] == (-2, 1, 1, 256)       # 224 workgroups would make 64-row bands of 512 KB
+    assert plan(1, 14336, 4096)[1:5] == (-2, 1, 1, 224)       # 256 KB bands: the whole-tile grid stands
+    assert plan(1, 16384, 16384)[1:5] == (-2, 1, 1, 256)      # 1 MB bands are fine with one tile per chunk
+
+
 def test_op_schemas_are_the_reference_schemas():
     import hf_rocm_kernels  # noqa: F401  (loads _HFRK_C)
     # the definition strings of the reference's csrc/torch_bindings.cpp:22,26-28,32-34,38-40, verbatim
