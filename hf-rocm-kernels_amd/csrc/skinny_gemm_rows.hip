@@ -1,4 +1,5 @@
-// FP8 skinny GEMM, m <= 16, weights of at least a few rows per workgroup: the row-split wave-stream kernel.
+// FP8 skinny GEMM, m <= 16 (up to 32 with a second activation tile), weights of at least a few rows per workgroup: the
+// row-split wave-stream kernel.
 //
 // Every workgroup owns a contiguous band of weight rows and all of K for them, so no sum ever crosses workgroups: there
 // is no workspace, no arrival counter and no memory round trip after the weight stream ends.  The weight rows are dealt
@@ -21,6 +22,11 @@
 //    precomputed bit mask says which), scales, rounds once and stores.  Each wave finishes at most one tile there.
 // Sums are added in wave order: results are bit-reproducible.
 //
+// Two things the host decides per launch: where in k a workgroup starts (rotated by its index when all waves of the launch
+// would otherwise read the same offset within 4 KB at every moment, GemmArgs::k_rotate), and how many workgroups there are
+// (the planner in skinny_gemm.hip: whole 16-row tiles where a grid of 224..256 gives them, twice the workgroups for short
+// bands at up to 4 rows, no bands of exactly 512 KB).
+//
 // Replaces, for these shapes, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and
 // consumers (producers/n_full_tiles.cu:4-127, consumers/mfma_16x16x32_consumer.cu:1-168,
 // consumers/smfma_16x16x64_consumer.cu:1-158).
@@ -39,6 +45,8 @@ __device__ __forceinline__ uint32_t pack16(float lo, float hi, bool bf16) {
 }
 
 // MA = ceil(m/4): 16-byte activation loads per lane and chunk (rows 4t .. 4t+3), RT = 16-row matrix tiles per chunk.
+// MA = 6 or 8 (17..32 rows, RT = 2, plain epilogue): the activation rows fill two 16-row tiles, and every weight operand
+// read from LDS feeds one matrix instruction per activation tile.
 // SWIGLU: the weight is a gate_up projection (gate rows [0, n/2), up rows [n/2, n)).  Bands, units and tiles then count
 // output columns (n/2 of them); a chunk pairs up to 16 gate rows with the up rows of the same columns (RT = 2: the gate
 // tile and the up tile), and the epilogue stores e4m3fn(silu(gate) * up / out_scale) into D [m, n/2] instead of the two
