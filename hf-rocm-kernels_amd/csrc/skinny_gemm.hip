@@ -766,11 +766,12 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
     // of L2 itself, which pays while a band's chunks stay large against them and k is moderate.  Measured against the
     // kernels below at 24 / 32 rows: 6144 x 4096 7.96 / 8.70 us against 9.54 / 9.55 (K-split, 1.5 tiles per workgroup),
     // 8192 x 8192 13.5 / 14.3 against 15.2 / 15.2, 10240 x 8192 18.5 against 19.4 at 24, 13312 x 16384 38.2 against 41.0 at
-    // 24, 16384 x 2048 8.9 against 10.3; slower on bands of 16 rows (4096 x 14336 +2 / +12 %), on k = 28672 (+3 / +7 %) and
-    // on the largest weights at 32 rows (57344 x 8192 +9 %).
+    // 24, 16384 x 2048 8.9 against 10.3, 8192 x 16384 26.5 against 31.7 at 32; slower on bands of 16 rows (4096 x 14336
+    // +2 / +12 %), on k = 28672 (+3 / +7 %), at 32 rows on bands of 40 rows and more with k = 16384 (+6 to +8 %) and on the
+    // largest weights (57344 x 8192 +9 %, 32768 x 8192 +16 %).
     if (m <= kRowsMaxM && !packed) {
         const long band_rows = 4 * (((long)(n + 3) / 4 + kNumCU - 1) / kNumCU);
-        const bool fits = m <= 24 ? (band_rows >= 24 && band_rows <= 64 && k <= 16384) : (band_rows >= 24 && band_rows <= 32 && k <= 8192);
+        const bool fits = band_rows >= 24 && band_rows <= (m <= 24 ? 64 : 32) && k <= 16384;
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
