@@ -717,7 +717,8 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 //   17 <= m <= 32    row-split kernel with two activation tiles on bands of 24-64 rows and moderate k (rule below)
 //   m  > 16          K-split kernel (activations in registers) when one window of it covers k; otherwise the
 //                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
-//                    4 row waves x 2 K waves almost everywhere; 2 x 4 for narrow weights (n <= 2048: more K parallelism
+//                    4 row waves x 2 K waves almost everywhere; 2 x 4 on long k (k >= 16384, n >= 8192, up to 48 rows) and
+//                    for narrow weights (n <= 2048: more K parallelism
 //                    where there are few row panels; from 2304 rows on 4 x 2 is 6-15 % faster, measured on 2304..5120 x
 //                    8192..16384 at m = 32, 48); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
 // workgroup decomposition with wn row waves x (8 / wn) K waves and ch chunks per slab, on min(256, units) workgroups
@@ -766,20 +767,24 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
     // of L2 itself, which pays while a band's chunks stay large against them and k is moderate.  Measured against the
     // kernels below at 24 / 32 rows: 6144 x 4096 7.96 / 8.70 us against 9.54 / 9.55 (K-split, 1.5 tiles per workgroup),
     // 8192 x 8192 13.5 / 14.3 against 15.2 / 15.2, 10240 x 8192 18.5 against 19.4 at 24, 13312 x 16384 38.2 against 41.0 at
-    // 24, 16384 x 2048 8.9 against 10.3, 8192 x 16384 26.5 against 31.7 at 32; slower on bands of 16 rows (4096 x 14336
-    // +2 / +12 %), on k = 28672 (+3 / +7 %), at 32 rows on bands of 40 rows and more with k = 16384 (+6 to +8 %) and on the
-    // largest weights (57344 x 8192 +9 %, 32768 x 8192 +16 %).
+    // 24, 16384 x 2048 8.9 against 10.3; slower on bands of 16 rows (4096 x 14336 +2 / +12 %), on k = 28672 (+3 / +7 %), at
+    // 32 rows with k = 16384 (8192 x 16384: 27.0 us against 25.3 for 2 row waves x 4 K waves below; bands of 40 rows and more
+    // +6 to +8 %) and on the largest weights (57344 x 8192 +9 %, 32768 x 8192 +16 %).
     if (m <= kRowsMaxM && !packed) {
         const long band_rows = 4 * (((long)(n + 3) / 4 + kNumCU - 1) / kNumCU);
         // (k = 2048 above 24 rows: the K-split kernel is 3-4 % ahead, 6144 x 2048 6.5 against 6.7 us)
-        const bool fits = band_rows >= 24 && band_rows <= (m <= 24 ? 64 : 32) && k <= 16384 && (m <= 24 || k >= 4096);
+        const bool fits = band_rows >= 24 && (m <= 24 ? (band_rows <= 64 && k <= 16384) : (band_rows <= 32 && k >= 4096 && k <= 8192));
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     const double weight_mb = (double)n * k / 1.0e6;
+    // 2 x 4 also on long k from 8192 rows on (k >= 16384, up to 48 activation rows: 8192 x 16384 25.3 against 27+ us at 32
+    // and 27.8 against 34.5 at 48; 10240 / 12288 / 16384 / 20480 / 24576 x 16384 at 32: 5-9 % faster; 13312 x 16384 equal).
+    // 8 x 1 from 220 MB on: 12288 x 16384 and 24576 x 8192 (201 MB) take 44.6 / 42.6 us with 4 x 2 against 50.3 / 47.0,
+    // 8192 x 28672 (235 MB) and 16384 x 16384 (268 MB) are 1-6 % faster with 8 x 1.
     int first = 4;
-    if (n <= 2048 && m <= 48) first = 2;
-    else if (weight_mb >= 200.0 && m > 48) first = 8;
+    if (m <= 48 && (n <= 2048 || (k >= 16384 && n >= 8192))) first = 2;
+    else if (weight_mb >= 220.0 && m > 48) first = 8;
     const int prefs[3][4] = {{2, 4, 1, 8}, {4, 2, 8, 1}, {8, 4, 2, 1}};
     const int* pref = first == 2 ? prefs[0] : first == 4 ? prefs[1] : prefs[2];
     for (int pi = 0; pi < 4; ++pi)

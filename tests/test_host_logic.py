@@ -267,7 +267,7 @@ def test_row_split_plans_for_17_to_32_rows_and_for_half_megabyte_bands():
     assert plan(24, 8192, 8192) == (0, -2, 2, 6, 256, 8 * 4 * 4096)
     assert plan(32, 8192, 8192) == (0, -2, 2, 8, 256, 8 * 4 * 4096)
     assert plan(20, 6144, 4096)[1:4] == (-2, 2, 6) and plan(32, 6144, 4096)[1:4] == (-2, 2, 8)
-    assert plan(32, 8192, 16384)[1:4] == (-2, 2, 8)
+    assert plan(32, 8192, 16384)[1:3] == (2, 4)  # 2 row waves x 4 K waves on long k
     assert plan(32, 10240, 8192)[1] != -2      # bands of 40 rows: up to 24 rows only
     assert plan(24, 4096, 14336)[1] != -2      # bands of 16 rows
     assert plan(24, 8192, 28672)[1] != -2      # k above 16384
