@@ -715,9 +715,10 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 //                    else the wave-stream kernel (chunk runs that may split a tile's k between workgroups); K-split kernel
 //                    for weights of at most 2048 chunks (8 MB) when one window of it covers k
 //   17 <= m <= 32    row-split kernel with two activation tiles on bands of 24-64 rows and moderate k (rule below)
-//   m  > 16          K-split kernel (activations in registers) when one window of it covers k; otherwise the
+//   m  > 16          workgroup kernel on whole row panels per workgroup where they deal out evenly (make_whole_panel_plan);
+//                    K-split kernel (activations in registers) when one window of it covers k; otherwise the
 //                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
-//                    4 row waves x 2 K waves almost everywhere; 2 x 4 on long k (k >= 16384, n >= 8192, up to 48 rows) and
+//                    4 row waves x 2 K waves almost everywhere; 2 x 4 on k = 16384 (n >= 8192, up to 48 rows) and
 //                    for narrow weights (n <= 2048: more K parallelism
 //                    where there are few row panels; from 2304 rows on 4 x 2 is 6-15 % faster, measured on 2304..5120 x
 //                    8192..16384 at m = 32, 48); 8 x 1 for 49+ rows on the largest weights (fewest reductions)
@@ -737,6 +738,43 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
     plan->slabs = k / ks;
     plan->lds_bytes = lds_bytes_for(mt, wk, ch);
     return HFRK_SUCCESS;
+}
+
+// 17+ rows: when the row panels of the workgroup kernel deal out evenly over 224..256 workgroups, every workgroup owns whole
+// panels and all of k for them -- no split of k between workgroups, no exchange at the end of the launch -- and the
+// activation slab is staged once for 8 waves.  The tallest panel that divides wins: 256 rows (8 row waves, two weight
+// tiles each), 128 (8 row waves) or 64 (4 row waves x 2 K waves).  Against the planner's other choice at 32 / 48 / 64 rows:
+// 57344 x 8192 (224 panels of 256 rows) 75.8 / 77.0 / 79.0 us against 79.8 / 84.3 / 91.1; 28672 x 8192 (224 of 128) 38.9 /
+// 40.8 / 42.5 against 43.9 / 46.2 / 55.8; 28672 x 4096 22.4 / 23.9 / 25.4 against 24.4 / 25.0 / 27.0 (K-split kernel);
+// 32768 x 4096 24.7 / 26.4 / 28.3 against 27.6 / 28.2 / 30.2; 16384 x 4096 (256 panels of 64) 14.3 / 15.7 / 17.4 against
+// 16.0 / 16.7 / 18.2; 14336 x 4096 (224 of 64) 13.5 / 14.9 / 16.5 against 15.3 / 15.9 / 17.1.
+static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    const int mt = (m + 15) / 16;
+    const int heights[3] = {256, 128, 64};
+    for (int hi = 0; hi < 3; ++hi) {
+        const int h = heights[hi];
+        if (n % h != 0) continue;
+        const long panels = n / h;
+        for (long g = kNumCU; g >= 7 * kNumCU / 8; g -= 8) {
+            if (panels % g != 0) continue;
+            const int wn = h == 64 ? 4 : 8, wk = kGemmWaves / wn, rt = h == 256 ? 2 : 1;
+            // two chunks per slab on short k with 8 row waves (28672 x 4096 at 64 rows: 25.4 against 26.5 us), else one
+            int ch = (wn == 8 && rt == 1 && k <= 5120 && k % 512 == 0) ? 2 : 1;
+            if (lds_bytes_for(mt, wk, ch, rt) > kLdsLimit) ch = 1;
+            const int ks = 256 * wk * ch;
+            if (k % ks != 0 || lds_bytes_for(mt, wk, ch, rt) > kLdsLimit || panels > kMaxPanels) continue;
+            plan->m_tiles = mt;
+            plan->wn = wn * rt;
+            plan->wk = wk;
+            plan->ch = ch;
+            plan->grid = (int)g;
+            plan->panels = (int)panels;
+            plan->slabs = k / ks;
+            plan->lds_bytes = lds_bytes_for(mt, wk, ch, rt);
+            return HFRK_SUCCESS;
+        }
+    }
+    return HFRK_INVALID_CONFIG;
 }
 
 static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = false) {
@@ -776,14 +814,16 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
         const bool fits = band_rows >= 24 && (m <= 24 ? (band_rows <= 64 && k <= 16384) : (band_rows <= 32 && k >= 4096 && k <= 8192));
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
+    if (make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     const double weight_mb = (double)n * k / 1.0e6;
-    // 2 x 4 also on long k from 8192 rows on (k >= 16384, up to 48 activation rows: 8192 x 16384 25.3 against 27+ us at 32
-    // and 27.8 against 34.5 at 48; 10240 / 12288 / 16384 / 20480 / 24576 x 16384 at 32: 5-9 % faster; 13312 x 16384 equal).
+    // 2 x 4 also on k = 16384 from 8192 rows on (up to 48 activation rows: 8192 x 16384 25.3 against 27+ us at 32 and 27.8
+    // against 34.5 at 48; 10240 / 12288 / 16384 / 20480 / 24576 x 16384 at 32: 5-9 % faster; 13312 x 16384 equal; not on
+    // k = 28672, where 8192 x 28672 takes 43.1 us with it against 39.9).
     // 8 x 1 from 220 MB on: 12288 x 16384 and 24576 x 8192 (201 MB) take 44.6 / 42.6 us with 4 x 2 against 50.3 / 47.0,
     // 8192 x 28672 (235 MB) and 16384 x 16384 (268 MB) are 1-6 % faster with 8 x 1.
     int first = 4;
-    if (m <= 48 && (n <= 2048 || (k >= 16384 && n >= 8192))) first = 2;
+    if (m <= 48 && (n <= 2048 || (k >= 16384 && k < 24576 && n >= 8192))) first = 2;
     else if (weight_mb >= 220.0 && m > 48) first = 8;
     const int prefs[3][4] = {{2, 4, 1, 8}, {4, 2, 8, 1}, {8, 4, 2, 1}};
     const int* pref = first == 2 ? prefs[0] : first == 4 ? prefs[1] : prefs[2];

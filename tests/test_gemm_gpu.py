@@ -104,13 +104,19 @@ def test_default_plan_matches_oracle(m, n, k):
     check_against_oracle(out, a, b, sa, sw)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 16384, 8192), (8, 8192, 16384), (5, 14336, 8192), (24, 8192, 8192), (32, 6144, 4096), (19, 16384, 2048)])
+@pytest.mark.parametrize("m,n,k", [(1, 16384, 8192), (8, 8192, 16384), (5, 14336, 8192), (24, 8192, 8192), (32, 6144, 4096), (19, 16384, 2048),
+                                   (33, 28672, 4096), (64, 57344, 8192), (40, 16384, 4096), (36, 14336, 4096), (48, 32768, 2048)])
 def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
-    """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224) and the 17..32
-    row variants of the row-split kernel, as the planner chooses them: against the oracle, plain and accumulating."""
+    """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), the 17..32 row
+    variants of the row-split kernel, and from 17 rows on the workgroup kernel on whole row panels per workgroup (256,
+    128 or 64 rows tall, on 224 or 256 workgroups), as the planner chooses them: against the oracle, plain and accumulating."""
     from hf_rocm_kernels import _capi
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
-    assert _capi.plan(m, n, k).wn == -2
+    p = _capi.plan(m, n, k)
+    if m <= 32 and n <= 16384:
+        assert p.wn == -2
+    else:
+        assert p.wn in (4, 8, 16) and (n // (16 * p.wn)) % p.grid == 0, p.as_dict()   # whole panels per workgroup
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k, per_token=True, per_channel=True)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     run_ex(a, b, sa, sw, out, accumulate=False)
