@@ -747,8 +747,10 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
 // 57344 x 8192 (224 panels of 256 rows) 75.8 / 77.0 / 79.0 us against 79.8 / 84.3 / 91.1; 28672 x 8192 (224 of 128) 38.9 /
 // 40.8 / 42.5 against 43.9 / 46.2 / 55.8; 28672 x 4096 22.4 / 23.9 / 25.4 against 24.4 / 25.0 / 27.0 (K-split kernel);
 // 32768 x 4096 24.7 / 26.4 / 28.3 against 27.6 / 28.2 / 30.2; 16384 x 4096 (256 panels of 64) 14.3 / 15.7 / 17.4 against
-// 16.0 / 16.7 / 18.2; 14336 x 4096 (224 of 64) 13.5 / 14.9 / 16.5 against 15.3 / 15.9 / 17.1.
+// 16.0 / 16.7 / 18.2; 14336 x 4096 (224 of 64) 13.5 / 14.9 / 16.5 against 15.3 / 15.9 / 17.1.  Up to k = 8192: on 16384 x
+// 16384 (a megabyte of weights per 64-row panel) the rules below are 6-7 % ahead.
 static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (k > 8192) return HFRK_INVALID_CONFIG;
     const int mt = (m + 15) / 16;
     const int heights[3] = {256, 128, 64};
     for (int hi = 0; hi < 3; ++hi) {
