@@ -728,12 +728,24 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
     if (k % ks != 0 || lds_bytes_for(mt, wk, ch) > kLdsLimit) return HFRK_INVALID_CONFIG;
     const long panels = (n + 16 * wn - 1) / (16 * wn);
     if (panels > kMaxPanels) return HFRK_BAD_SHAPE;
-    const long units = panels * (k / ks);
+    const long slabs = k / ks, units = panels * slabs;
+    // Small weights (a workgroup's run of units shorter than a panel): a grid under which every run is a whole fraction of
+    // a panel.  Runs that straddle panel boundaries add contributors to both panels' exchanges (3072 x 8192 at 32 / 64
+    // rows: 768 units are 3 per workgroup on 256, cutting the 16-slab panels unevenly, 12.1 / 15.0 us; 4 per workgroup on
+    // 192, 9.8 / 12.4 us; 6144 x 5120 at 64 rows: 17.8 on 256, 15.0 on 192).  Down to 192 workgroups; longer runs keep the
+    // full grid (20480 x 8192: 36.0 us on 160 workgroups with whole panels against 34.6 on 256).
+    long grid = units < kNumCU ? units : kNumCU;
+    if (units > kNumCU)
+        for (long g = kNumCU; g >= 3 * kNumCU / 4; g -= 8) {
+            if (units % g != 0) continue;
+            const long per = units / g;
+            if (per < slabs && slabs % per == 0) { grid = g; break; }
+        }
     plan->m_tiles = mt;
     plan->wn = wn;
     plan->wk = wk;
     plan->ch = ch;
-    plan->grid = (int)(units < kNumCU ? units : kNumCU);
+    plan->grid = (int)grid;
     plan->panels = (int)panels;
     plan->slabs = k / ks;
     plan->lds_bytes = lds_bytes_for(mt, wk, ch);
@@ -749,19 +761,45 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
 // 32768 x 4096 24.7 / 26.4 / 28.3 against 27.6 / 28.2 / 30.2; 16384 x 4096 (256 panels of 64) 14.3 / 15.7 / 17.4 against
 // 16.0 / 16.7 / 18.2; 14336 x 4096 (224 of 64) 13.5 / 14.9 / 16.5 against 15.3 / 15.9 / 17.1.  Up to k = 8192: on 16384 x
 // 16384 (a megabyte of weights per 64-row panel) the rules below are 6-7 % ahead.
+// One panel per workgroup also on 160..216 workgroups: idle compute units cost in proportion to the bytes, the exchange
+// they save does not, and the other rules' deal over 256 is uneven for such row counts.  At 32 / 48 / 64 rows, against the
+// rules below:
+//   64-row panels, the shorter k the fewer workgroups: 10240 rows on 160 workgroups 10.0 / 11.5 / 12.9 us against 13.7 / 16.4 /
+//   17.7 at k = 3072 and 14.9 / 16.9 / 18.5 against 16.4 / 18.7 / 20.1 at 5120, level at 8192, 4-11 % behind at 14336; 12288
+//   rows on 192: 26-30 % ahead at 3072, 5-10 % at 8192 (level at 64 rows), level at 14336; 13312 rows on 208: 28-36 % ahead
+//   at 3072, 22-29 % at 8192, 13-17 % at 14336, level at 16384.  At k = 4096 the K-split kernel is 4-8 % ahead of 160 / 192
+//   such workgroups from 33 rows on;
+//   128-row panels (taken first): 24576 rows on 192 workgroups 16.0 / 17.7 / 18.8 against 18.8 / 21.7 / 23.9 at k = 3072, 35.0
+//   / 37.8 / 39.9 against 36.3 / 39.9 / 43.1 at 8192, 64.2 / 68.1 / 71.5 against 70.5 / 78.3 / 82.4 at 16384 (level at 14336);
+//   20480 rows on 160: 15.0 / 16.7 / 17.8 against 17.3 / 19.7 / 21.3 at 3072, 32.4 / 35.4 / 37.4 against 34.4 / 36.7 / 38.3
+//   at 8192, behind from 14336 on and behind the K-split kernel at 4096;
+//   k = 16384 up to 48 rows: 64-row panels with two chunks per slab, 14336 rows on 224 workgroups 41.9 / 43.7 us against 44.9
+//   / 49.8, 16384 rows on 256 46.8 / 48.5 against 47.4 / 52.2 (with one chunk per slab it is 6-7 % behind there).
 static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
-    if (k > 8192) return HFRK_INVALID_CONFIG;
     const int mt = (m + 15) / 16;
     const int heights[3] = {256, 128, 64};
     for (int hi = 0; hi < 3; ++hi) {
         const int h = heights[hi];
         if (n % h != 0) continue;
         const long panels = n / h;
-        for (long g = kNumCU; g >= 7 * kNumCU / 8; g -= 8) {
-            if (panels % g != 0) continue;
+        long g_try[2] = {0, 0};  // several panels each on 224..256 workgroups; one panel each on fewer
+        if (k <= 8192)
+            for (long g = kNumCU; g >= 7 * kNumCU / 8 && !g_try[0]; g -= 8)
+                if (panels % g == 0) g_try[0] = g;
+        if (h == 64 && k == 16384 && m <= 48 && panels == kNumCU) g_try[0] = panels;
+        if (panels % 8 == 0 && panels < kNumCU) {
+            bool one_each = false;
+            if (h == 64) one_each = panels >= (k <= 5120 ? 160 : k <= 8192 ? 192 : 208) && k <= 14336 && !(k == 4096 && m > 32 && panels < 208);
+            if (h == 64 && k == 16384 && m <= 48) one_each = panels >= 208;
+            if (h == 128) one_each = panels >= 192 || (panels >= 160 && k <= 8192 && k != 4096 && k != 2048);
+            if (one_each) g_try[1] = panels;
+        }
+        for (int gi = 0; gi < 2; ++gi) {
+            const long g = g_try[gi];
+            if (g == 0) continue;
             const int wn = h == 64 ? 4 : 8, wk = kGemmWaves / wn, rt = h == 256 ? 2 : 1;
             // two chunks per slab on short k with 8 row waves (28672 x 4096 at 64 rows: 25.4 against 26.5 us), else one
-            int ch = (wn == 8 && rt == 1 && k <= 5120 && k % 512 == 0) ? 2 : 1;
+            int ch = ((wn == 8 && rt == 1 && k <= 5120 && k % 512 == 0) || (wn == 4 && k > 14336)) ? 2 : 1;
             if (lds_bytes_for(mt, wk, ch, rt) > kLdsLimit) ch = 1;
             const int ks = 256 * wk * ch;
             if (k % ks != 0 || lds_bytes_for(mt, wk, ch, rt) > kLdsLimit || panels > kMaxPanels) continue;
@@ -775,6 +813,24 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
             plan->lds_bytes = lds_bytes_for(mt, wk, ch, rt);
             return HFRK_SUCCESS;
         }
+    }
+    return HFRK_INVALID_CONFIG;
+}
+
+// Long k (14336, 16384): 128-row panels, 8 row waves, each panel's k cut between 2 or 4 workgroups, on the 192..256
+// workgroups that makes.  Against the other rules at 32 / 48 / 64 rows: 6144 x 16384 (4 x 48 panels) 21.5 / 24.3 / 25.8 us
+// against 25.3 / 28.4 / 30.4 and 5-7 % ahead at k = 14336; 13312 x 16384 (2 x 104) 39.7 / 42.0 / 45.0 against 42.8 / 48.1 /
+// 50.1; 12288 x 16384 (2 x 96) 3-5 % ahead; 8192 x 16384 (4 x 64) 29.8 against 35.9 at 64 rows, but 3-4 % behind 2 row
+// waves x 4 K waves up to 48 rows, so all 256 workgroups only from 49 rows on.
+static int make_split_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (k < 14336 || k > 16384 || n % 128 != 0) return HFRK_INVALID_CONFIG;
+    const long panels = n / 128, slabs = k / 256;
+    for (int f = 2; f <= 4; f += 2) {
+        const long g = panels * f;
+        if (g < 3 * kNumCU / 4 || g > kNumCU || g % 8 != 0 || slabs % f != 0 || (g == kNumCU && m <= 48)) continue;
+        if (fill_workgroup_plan(m, n, k, 8, 1, plan) != HFRK_SUCCESS) return HFRK_INVALID_CONFIG;
+        plan->grid = (int)g;
+        return HFRK_SUCCESS;
     }
     return HFRK_INVALID_CONFIG;
 }
@@ -810,13 +866,22 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
     // 24, 16384 x 2048 8.9 against 10.3; slower on bands of 16 rows (4096 x 14336 +2 / +12 %), on k = 28672 (+3 / +7 %), at
     // 32 rows with k = 16384 (8192 x 16384: 27.0 us against 25.3 for 2 row waves x 4 K waves below; bands of 40 rows and more
     // +6 to +8 %) and on the largest weights (57344 x 8192 +9 %, 32768 x 8192 +16 %).
+    // Bands of 12-20 rows (3072..5120 weight rows) on k up to 8192 as well, where the kernels below deal their units
+    // unevenly: 5120 x 5120 8.95 / 9.2 / 9.9 / 10.1 us at 20 / 24 / 28 / 32 rows against 11.3-11.6, 3072 x 3072 6.7 / 6.8 /
+    // 7.3 / 7.35 against 8.5, 4096 x 5120 8.4 / 8.5 / 9.2 / 9.35 against 9.8-9.9, 5120 x 8192 11.0 / 11.3 / 12.1 / 12.4 against
+    // 13.7-13.8.  Not where one K-split window covers k and its tiles deal out evenly (3072 and 4096 rows at k = 2048 and
+    // 4096: level or 0.3-0.9 us behind), nor above 24 rows at k = 8192 on bands under 20 rows or at k = 2048.
     if (m <= kRowsMaxM && !packed) {
         const long band_rows = 4 * (((long)(n + 3) / 4 + kNumCU - 1) / kNumCU);
         // (k = 2048 above 24 rows: the K-split kernel is 3-4 % ahead, 6144 x 2048 6.5 against 6.7 us)
-        const bool fits = band_rows >= 24 && (m <= 24 ? (band_rows <= 64 && k <= 16384) : (band_rows <= 32 && k >= 4096 && k <= 8192));
+        bool fits = band_rows >= 24 && (m <= 24 ? (band_rows <= 64 && k <= 16384) : (band_rows <= 32 && k >= 3072 && k <= 8192));
+        if (band_rows >= 12 && band_rows < 24 && k >= (m <= 24 ? 2048 : 3072) && k <= 8192)
+            fits = ((k != 2048 && k != 4096) || band_rows >= 20) && (m <= 24 || k < 8192 || band_rows >= 20);
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
+    if (k >= 16384 && make_split_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
+    if (make_split_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     const double weight_mb = (double)n * k / 1.0e6;
     // 2 x 4 also on k = 16384 from 8192 rows on (up to 48 activation rows: 8192 x 16384 25.3 against 27+ us at 32 and 27.8

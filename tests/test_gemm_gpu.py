@@ -105,18 +105,23 @@ def test_default_plan_matches_oracle(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 16384, 8192), (8, 8192, 16384), (5, 14336, 8192), (24, 8192, 8192), (32, 6144, 4096), (19, 16384, 2048),
-                                   (33, 28672, 4096), (64, 57344, 8192), (40, 16384, 4096), (36, 14336, 4096), (48, 32768, 2048)])
+                                   (33, 28672, 4096), (64, 57344, 8192), (40, 16384, 4096), (36, 14336, 4096), (48, 32768, 2048),
+                                   (20, 5120, 5120), (32, 3072, 3072), (28, 4096, 5120), (64, 10240, 3072), (48, 12288, 8192),
+                                   (33, 13312, 14336), (48, 24576, 16384), (64, 20480, 3072), (40, 16384, 16384),
+                                   (48, 13312, 16384), (32, 6144, 16384), (64, 8192, 16384), (17, 6144, 14336)])
 def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
     """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), the 17..32 row
     variants of the row-split kernel, and from 17 rows on the workgroup kernel on whole row panels per workgroup (256,
-    128 or 64 rows tall, on 224 or 256 workgroups), as the planner chooses them: against the oracle, plain and accumulating."""
+    128 or 64 rows tall, on 160 to 256 workgroups, or 128-row panels whose k is cut between 2 or 4 workgroups), as the planner
+    chooses them: against the oracle, plain and accumulating."""
     from hf_rocm_kernels import _capi
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     p = _capi.plan(m, n, k)
-    if m <= 32 and n <= 16384:
+    if m <= 32 and n <= 16384 and (k <= 8192 or m <= 24):
         assert p.wn == -2
     else:
-        assert p.wn in (4, 8, 16) and (n // (16 * p.wn)) % p.grid == 0, p.as_dict()   # whole panels per workgroup
+        panels = n // (16 * p.wn)
+        assert p.wn in (4, 8, 16) and (panels % p.grid == 0 or p.grid % panels == 0), p.as_dict()   # whole panels, or whole fractions
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k, per_token=True, per_channel=True)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     run_ex(a, b, sa, sw, out, accumulate=False)

@@ -280,6 +280,38 @@ def test_row_split_plans_for_17_to_32_rows_and_for_half_megabyte_bands():
     assert plan(1, 14336, 8192)[1:5] == (-2, 1, 1, 256)       # 224 workgroups would make 64-row bands of 512 KB
     assert plan(1, 14336, 4096)[1:5] == (-2, 1, 1, 224)       # 256 KB bands: the whole-tile grid stands
     assert plan(1, 16384, 16384)[1:5] == (-2, 1, 1, 256)      # 1 MB bands are fine with one tile per chunk
+    # bands of 12-20 rows on k up to 8192, except where one K-split window covers k and its tiles deal out evenly
+    assert plan(20, 5120, 5120)[1:4] == (-2, 2, 6) and plan(32, 3072, 3072)[1:4] == (-2, 2, 8)
+    assert plan(24, 5120, 4096)[1] == -2 and plan(24, 4096, 4096)[1] == -1
+    assert plan(32, 4096, 8192)[1] > 0 and plan(24, 4096, 8192)[1] == -2
+
+
+def test_workgroup_plans_on_whole_and_split_panels():
+    """From 17 rows on the planner deals whole row panels to workgroups where the row count allows: several each on
+    224..256 workgroups, one each on 160..216 (64-row panels on short k, 128-row panels), and on long k 128-row panels
+    whose k is cut between 2 or 4 workgroups."""
+    p = _capi.GemmPlan()
+    lib = _capi.load()
+    plan = lambda m, n, k: (lib.hfrk_skinny_gemm_plan(m, n, k, ctypes.byref(p)), p.wn, p.wk, p.ch, p.grid, p.panels)
+    assert plan(64, 57344, 8192)[1:6] == (16, 1, 1, 224, 224)
+    assert plan(48, 28672, 4096)[1:6] == (8, 1, 2, 224, 224)
+    assert plan(40, 16384, 4096)[1:6] == (4, 2, 1, 256, 256)
+    # one panel per workgroup on fewer workgroups
+    assert plan(64, 10240, 3072)[1:6] == (4, 2, 1, 160, 160)
+    assert plan(64, 10240, 8192)[4] == 256                      # too much k for 160 workgroups
+    assert plan(48, 12288, 8192)[1:6] == (4, 2, 1, 192, 192)
+    assert plan(33, 13312, 14336)[1:6] == (4, 2, 1, 208, 208)
+    assert plan(48, 12288, 4096)[1] == -1 and plan(32, 12288, 4096)[1:6] == (4, 2, 1, 192, 192)
+    assert plan(48, 24576, 16384)[1:6] == (8, 1, 1, 192, 192)
+    assert plan(64, 20480, 3072)[1:6] == (8, 1, 2, 160, 160)
+    assert plan(64, 20480, 4096)[1] == -1 and plan(64, 20480, 14336)[4] == 256
+    # k = 16384: 64-row panels with two chunks per slab up to 48 rows; 128-row panels cut in k
+    assert plan(40, 16384, 16384)[1:6] == (4, 2, 2, 256, 256)
+    assert plan(64, 16384, 16384)[1:3] == (8, 1)
+    assert plan(48, 13312, 16384)[1:6] == (8, 1, 1, 208, 104)
+    assert plan(32, 6144, 16384)[1:6] == (8, 1, 1, 192, 48)
+    assert plan(32, 6144, 14336)[1:6] == (8, 1, 1, 192, 48)
+    assert plan(48, 8192, 16384)[1:3] == (2, 4) and plan(64, 8192, 16384)[1:6] == (8, 1, 1, 256, 64)
 
 
 def test_op_schemas_are_the_reference_schemas():
