@@ -714,7 +714,8 @@ static int make_ksplit_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 //   m <= 16          row-split kernel (a band of weight rows and all of k per workgroup) when the rows deal out evenly,
 //                    else the wave-stream kernel (chunk runs that may split a tile's k between workgroups); K-split kernel
 //                    for weights of at most 2048 chunks (8 MB) when one window of it covers k
-//   17 <= m <= 32    row-split kernel with two activation tiles on bands of 24-64 rows and moderate k (rule below)
+//   17 <= m <= 32    row-split kernel with two activation tiles on bands of 12-64 rows and moderate k (rule below), behind
+//                    whole 64-row panels of the workgroup kernel from 12288 weight rows on
 //   m  > 16          workgroup kernel on whole row panels per workgroup where they deal out evenly (make_whole_panel_plan);
 //                    K-split kernel (activations in registers) when one window of it covers k; otherwise the
 //                    workgroup kernel, which stages the activation slab once per workgroup in LDS:
@@ -786,6 +787,7 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         if (k <= 8192)
             for (long g = kNumCU; g >= 7 * kNumCU / 8 && !g_try[0]; g -= 8)
                 if (panels % g == 0) g_try[0] = g;
+        if (h == 64 && k > 8192 && k <= 14336 && panels == kNumCU) g_try[0] = panels;  // (what the rules below choose from 25 rows on)
         if (h == 64 && k == 16384 && m <= 48 && panels == kNumCU) g_try[0] = panels;
         if (panels % 8 == 0 && panels < kNumCU) {
             bool one_each = false;
@@ -877,6 +879,10 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
         bool fits = band_rows >= 24 && (m <= 24 ? (band_rows <= 64 && k <= 16384) : (band_rows <= 32 && k >= 3072 && k <= 8192));
         if (band_rows >= 12 && band_rows < 24 && k >= (m <= 24 ? 2048 : 3072) && k <= 8192)
             fits = ((k != 2048 && k != 4096) || band_rows >= 20) && (m <= 24 || k < 8192 || band_rows >= 20);
+        // From 12288 weight rows on, whole 64-row panels per workgroup come first where they exist: at 20 / 24 rows 12288 x
+        // 8192 19.8 / 20.0 us against 20.5 / 21.2, 13312 x 8192 20.6 / 20.8 against 21.7 / 22.2, 14336 x 5120 15.7 / 15.8 against
+        // 17.2 / 17.7, 16384 x 14336 39.4 / 39.2 against 42.1 / 43.3; level at k = 4096 and 16384 and on 10240 rows.
+        if (fits && band_rows >= 48 && k != 2048 && k < 16384 && make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
     if (k >= 16384 && make_split_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;

@@ -108,7 +108,8 @@ def test_default_plan_matches_oracle(m, n, k):
                                    (33, 28672, 4096), (64, 57344, 8192), (40, 16384, 4096), (36, 14336, 4096), (48, 32768, 2048),
                                    (20, 5120, 5120), (32, 3072, 3072), (28, 4096, 5120), (64, 10240, 3072), (48, 12288, 8192),
                                    (33, 13312, 14336), (48, 24576, 16384), (64, 20480, 3072), (40, 16384, 16384),
-                                   (48, 13312, 16384), (32, 6144, 16384), (64, 8192, 16384), (17, 6144, 14336)])
+                                   (48, 13312, 16384), (32, 6144, 16384), (64, 8192, 16384), (17, 6144, 14336),
+                                   (20, 14336, 5120), (24, 16384, 14336), (18, 13312, 8192)])
 def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
     """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), the 17..32 row
     variants of the row-split kernel, and from 17 rows on the workgroup kernel on whole row panels per workgroup (256,
@@ -117,7 +118,7 @@ def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
     from hf_rocm_kernels import _capi
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     p = _capi.plan(m, n, k)
-    if m <= 32 and n <= 16384 and (k <= 8192 or m <= 24):
+    if m <= 16 or (m <= 32 and (n <= 8192 or k == 2048) and (k <= 8192 or m <= 24)):
         assert p.wn == -2
     else:
         panels = n // (16 * p.wn)

@@ -312,6 +312,9 @@ def test_workgroup_plans_on_whole_and_split_panels():
     assert plan(32, 6144, 16384)[1:6] == (8, 1, 1, 192, 48)
     assert plan(32, 6144, 14336)[1:6] == (8, 1, 1, 192, 48)
     assert plan(48, 8192, 16384)[1:3] == (2, 4) and plan(64, 8192, 16384)[1:6] == (8, 1, 1, 256, 64)
+    # 17..24 rows: whole 64-row panels come before the row-split kernel from 12288 weight rows on
+    assert plan(24, 13312, 8192)[1:6] == (4, 2, 1, 208, 208) and plan(20, 16384, 14336)[1:6] == (4, 2, 1, 256, 256)
+    assert plan(24, 10240, 8192)[1] == -2 and plan(19, 16384, 2048)[1] == -2 and plan(24, 16384, 16384)[1] == -2
 
 
 def test_op_schemas_are_the_reference_schemas():
