@@ -663,7 +663,18 @@ static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     // that would create such bands is not taken for the sake of whole tiles (14336 x 8192: 22.4 us on 224 workgroups,
     // 19.4 on 256).
     auto half_mb_bands = [&](long g) { return units % g == 0 && 4 * (units / g) * (long)k == (1L << 19); };
-    if (units % (4 * grid) != 0) {
+    // Bands of 20..44 rows that are no multiple of 16 cut into one or two chunks per 256 bytes of k with two matrix tiles per
+    // chunk instead of two or three (20 rows: one 5 KB chunk instead of 3 + 2 KB), which pays from 5 rows on once k is long
+    // enough: 5120 x 8192 9.3 against 9.7 us at 8 rows and 9.8 against 11.1 at 16, 5120 x 16384 15.9 / 16.6 against 16.9 / 19.3,
+    // 10240 x 8192 15.8 against 16.3 at 8, 11264 x 16384 31.0 against 32.4; at k = 5120 from 9 rows on (5120 x 5120 at 16: 7.9
+    // against 8.5) and below on bands of 36+ rows (10240 x 5120 at 8: 11.1 against 11.6; 6144 x 5120 8.0 against 7.8 the other
+    // way); level at k = 3072 and on bands of 52 rows (13312 x 16384).
+    // On long k such bands also beat a smaller grid of whole tiles (7168 x 14336 at 8 rows: 18.1 us on 256 against 19.2 on 224).
+    auto ragged = [&](long band) {
+        if (m < 5) return band == 20 && k >= 8192;  // (5120 x 8192 / 14336 / 16384 at 1 row: 9.0 / 13.7 / 15.6 us against 9.4 / 14.3 / 16.3 on 512 workgroups)
+        return band > 16 && band <= 48 && band % 16 != 0 && (k >= 8192 || (k >= 5120 && (band >= 36 || m >= 9)));
+    };
+    if (units % (4 * grid) != 0 && !(k >= 8192 && ragged(4 * busiest))) {
         long whole = 0;
         for (long g = kNumCU - 8; g >= 7 * kNumCU / 8; g -= 8)
             if (units % (4 * g) == 0 && !half_mb_bands(g)) { whole = g; break; }
@@ -671,7 +682,8 @@ static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         else if (m <= 4 && 4 * busiest <= 48 && units >= 4 * kNumCU) grid = 2 * kNumCU;  // bands of at least 8 rows
     }
     const long rows_per_band = 4 * ((units + grid - 1) / grid);
-    const int row_tiles = (m > 16 || (m >= 9 && rows_per_band >= 24) || (half_mb_bands(grid) && rows_per_band >= 24)) ? 2 : 1;
+    const bool ragged_band = ragged(rows_per_band) && (m >= 5 || grid == kNumCU);
+    const int row_tiles = (m > 16 || (m >= 9 && rows_per_band >= 24) || (half_mb_bands(grid) && rows_per_band >= 24) || ragged_band) ? 2 : 1;
     return fill_rows_plan(m, n, k, row_tiles, (int)grid, plan);
 }
 

@@ -109,9 +109,11 @@ def test_default_plan_matches_oracle(m, n, k):
                                    (20, 5120, 5120), (32, 3072, 3072), (28, 4096, 5120), (64, 10240, 3072), (48, 12288, 8192),
                                    (33, 13312, 14336), (48, 24576, 16384), (64, 20480, 3072), (40, 16384, 16384),
                                    (48, 13312, 16384), (32, 6144, 16384), (64, 8192, 16384), (17, 6144, 14336),
-                                   (20, 14336, 5120), (24, 16384, 14336), (18, 13312, 8192)])
+                                   (20, 14336, 5120), (24, 16384, 14336), (18, 13312, 8192),
+                                   (8, 5120, 8192), (4, 5120, 8192), (16, 5120, 5120), (7, 7168, 14336), (5, 11264, 5120)])
 def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
-    """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), the 17..32 row
+    """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), ragged bands of
+    20..44 rows (two weight tiles per chunk from 5 rows on), the 17..32 row
     variants of the row-split kernel, and from 17 rows on the workgroup kernel on whole row panels per workgroup (256,
     128 or 64 rows tall, on 160 to 256 workgroups, or 128-row panels whose k is cut between 2 or 4 workgroups), as the planner
     chooses them: against the oracle, plain and accumulating."""

@@ -280,6 +280,13 @@ def test_row_split_plans_for_17_to_32_rows_and_for_half_megabyte_bands():
     assert plan(1, 14336, 8192)[1:5] == (-2, 1, 1, 256)       # 224 workgroups would make 64-row bands of 512 KB
     assert plan(1, 14336, 4096)[1:5] == (-2, 1, 1, 224)       # 256 KB bands: the whole-tile grid stands
     assert plan(1, 16384, 16384)[1:5] == (-2, 1, 1, 256)      # 1 MB bands are fine with one tile per chunk
+    # ragged bands of 20..44 rows: two matrix tiles per chunk from 5 rows on, on long enough k; 256 workgroups rather than
+    # fewer with whole tiles
+    assert plan(8, 5120, 8192)[1:5] == (-2, 2, 2, 256) and plan(4, 5120, 8192)[1:5] == (-2, 2, 1, 256) and plan(4, 5120, 4096)[1:5] == (-2, 1, 1, 512)
+    assert plan(4, 10240, 8192)[2] == 1 and plan(8, 5120, 5120)[2] == 1
+    assert plan(16, 5120, 5120)[1:5] == (-2, 2, 4, 256) and plan(8, 10240, 5120)[2] == 2 and plan(8, 13312, 16384)[2] == 1
+    assert plan(8, 7168, 14336)[1:5] == (-2, 2, 2, 256) and plan(8, 7168, 4096)[1:5] == (-2, 1, 2, 224)
+    assert plan(8, 6144, 4096)[1:5] == (-2, 1, 2, 256)
     # bands of 12-20 rows on k up to 8192, except where one K-split window covers k and its tiles deal out evenly
     assert plan(20, 5120, 5120)[1:4] == (-2, 2, 6) and plan(32, 3072, 3072)[1:4] == (-2, 2, 8)
     assert plan(24, 5120, 4096)[1] == -2 and plan(24, 4096, 4096)[1] == -1
