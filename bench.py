@@ -77,8 +77,8 @@ WORKLOADS = {
         "text": "llama3-70b decode linears: M in {1,4,8,16,32} x qkv(10240,8192) o_proj(8192,8192) gate_up(57344,8192) "
                 "down(8192,28672); FP8 e4m3fn A and W, per-tensor scales, bf16 out; 20 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s over Llama-3-70B decode shapes, M=1..32 (us/call in `cases`)",
-        "kernel": "hfrk::skinny_gemm_rows_kernel (M<=16, and o_proj at M=32), hfrk::skinny_gemm_kernel<2,4,2,1,1> (M=32: gate_up, "
-                  "down), hfrk::skinny_gemm_ksplit_kernel<2,1024> (M=32: qkv, by plan table)",
+        "kernel": "hfrk::skinny_gemm_rows_kernel (M<=16, and o_proj at M=32), hfrk::skinny_gemm_kernel<2,8,1,1,2> (M=32: gate_up, whole "
+                  "256-row panels), <2,4,2,1,1> (M=32: down), hfrk::skinny_gemm_ksplit_kernel<2,1024> (M=32: qkv, by plan table)",
     },
     "scaled-m": {
         "shapes": [("o_proj", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336)],
@@ -87,7 +87,7 @@ WORKLOADS = {
                 "(rows 1 and M-1 are 20x outliers) and per-output-channel weight scales, bf16 out; 9 calls per step",
         "metric": "FP8 skinny-GEMM achieved HBM GB/s, per-token x per-channel scales, M=16..64 (us/call in `cases`)",
         "kernel": "hfrk::skinny_gemm_rows_kernel (M=16), hfrk::skinny_gemm_ksplit_kernel (M=32,64 on K=4096), "
-                  "hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64 on K=14336 and plan-table entries)",
+                  "hfrk::skinny_gemm_kernel<MT,WN,WK,CH> (M=32,64: whole 128-row panels on (28672,4096), 4 x 2 waves on K=14336)",
     },
     "llama31-405b-tp8": {
         "shapes": [("o_proj", 16384, 2048), ("qkv", 2304, 16384), ("gate_up", 13312, 16384), ("down", 16384, 6656)],
