@@ -544,11 +544,12 @@ def test_plan_table_overrides_the_planner_and_round_trips_through_a_file(tmp_pat
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (16, 28672, 4096), (32, 4096, 14336), (64, 8192, 8192),
-                                   (40, 1000, 2048), (17, 50, 256)])
+                                   (40, 1000, 2048), (17, 50, 256), (4, 2048, 2048), (4, 2048, 4096), (4, 2048, 28672)])
 def test_every_plan_the_sweep_tool_proposes_is_one_the_library_accepts(m, n, k):
     """benchmarks/skinny_gemm/grid_search.py enumerates hfrk_gemm_plan structs by its own arithmetic; the library
     validates plans with its own (hfrk_plan_table_set runs the launcher's check, no device needed).  They must agree,
-    for every decomposition family, and describe() must name each one."""
+    for every decomposition family, and describe() must name each one.  Every accepted plan also goes through the host-side
+    restatement of its kernel's index arithmetic: every unit of work covered exactly once, ranges contiguous."""
     from hf_rocm_kernels import plan_table
     from hf_rocm_kernels.benchmarks.skinny_gemm import grid_search
     plans = grid_search.candidate_plans(m, n, k, [7, 160, 224, 256, 512])
@@ -560,6 +561,15 @@ def test_every_plan_the_sweep_tool_proposes_is_one_the_library_accepts(m, n, k):
             status = _capi.load().hfrk_plan_table_set(m, n, k, 0, ctypes.byref(p))
             assert status == _capi.SUCCESS, (grid_search.describe(p), p.as_dict(), _capi.status_string(status))
             families.add(grid_search.describe(p).split()[0])
+            if p.wn == -2:
+                _emulate_rows(p)
+            elif p.wn == 0:
+                assert all(c == 1 for c in _emulate_stream(p)[0]), grid_search.describe(p)
+            elif p.wn == -1:
+                r = _stream_ranges(p)
+                assert r[0][0] == 0 and r[-1][1] == p.panels * p.slabs and all(a[1] == b[0] for a, b in zip(r, r[1:]))
+            else:
+                assert all(c == 1 for row in _emulate(p, n, k)[0] for c in row), grid_search.describe(p)
     finally:
         plan_table.clear()
     assert "workgroup" in families
