@@ -788,7 +788,7 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
 //   at 8192, behind from 14336 on and behind the K-split kernel at 4096;
 //   k = 16384 up to 48 rows: 64-row panels with two chunks per slab, 14336 rows on 224 workgroups 41.9 / 43.7 us against 44.9
 //   / 49.8, 16384 rows on 256 46.8 / 48.5 against 47.4 / 52.2 (with one chunk per slab it is 6-7 % behind there).
-static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = false) {
     const int mt = (m + 15) / 16;
     const int heights[3] = {256, 128, 64};
     for (int hi = 0; hi < 3; ++hi) {
@@ -799,13 +799,17 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
         if (k <= 8192)
             for (long g = kNumCU; g >= 7 * kNumCU / 8 && !g_try[0]; g -= 8)
                 if (panels % g == 0) g_try[0] = g;
-        if (h == 64 && k > 8192 && k <= 14336 && panels == kNumCU) g_try[0] = panels;  // (what the rules below choose from 25 rows on)
+        // (what the rules below choose from 25 rows on; at 64 rows 8 row waves are 3 % ahead on 16384 x 14336)
+        if (h == 64 && k > 8192 && k <= 14336 && panels == kNumCU && m <= 48) g_try[0] = panels;
         if (h == 64 && k == 16384 && m <= 48 && panels == kNumCU) g_try[0] = panels;
         if (panels % 8 == 0 && panels < kNumCU) {
             bool one_each = false;
             if (h == 64) one_each = panels >= (k <= 5120 ? 160 : k <= 8192 ? 192 : 208) && k <= 14336 && !(k == 4096 && m > 32 && panels < 208);
             if (h == 64 && k == 16384 && m <= 48) one_each = panels >= 208;
             if (h == 128) one_each = panels >= 192 || (panels >= 160 && k <= 8192 && k != 4096 && k != 2048);
+            // (packed weights, 24576 x 8192: 42.0 / 41.9 / 45.2 us at 20 / 32 / 64 rows against 36.4 / 36.6 / 43.2 for the rules
+            // below -- a panel is 1 MB of contiguous bytes there; k = 3072, 5120 and 16384 gain 11-24 % in both layouts)
+            if (h == 128 && packed && k == 8192) one_each = false;
             if (one_each) g_try[1] = panels;
         }
         for (int gi = 0; gi < 2; ++gi) {
@@ -836,12 +840,12 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
 // against 25.3 / 28.4 / 30.4 and 5-7 % ahead at k = 14336; 13312 x 16384 (2 x 104) 39.7 / 42.0 / 45.0 against 42.8 / 48.1 /
 // 50.1; 12288 x 16384 (2 x 96) 3-5 % ahead; 8192 x 16384 (4 x 64) 29.8 against 35.9 at 64 rows, but 3-4 % behind 2 row
 // waves x 4 K waves up to 48 rows, so all 256 workgroups only from 49 rows on.
-static int make_split_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+static int make_split_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed) {
     if (k < 14336 || k > 16384 || n % 128 != 0) return HFRK_INVALID_CONFIG;
     const long panels = n / 128, slabs = k / 256;
     for (int f = 2; f <= 4; f += 2) {
         const long g = panels * f;
-        if (g < 3 * kNumCU / 4 || g > kNumCU || g % 8 != 0 || slabs % f != 0 || (g == kNumCU && m <= 48)) continue;
+        if (g < 3 * kNumCU / 4 || g > kNumCU || g % 8 != 0 || slabs % f != 0 || (g == kNumCU && (m <= 48 || packed))) continue;  // (packed 8192 x 16384 at 64 rows: 30.6 us against 29.6)
         if (fill_workgroup_plan(m, n, k, 8, 1, plan) != HFRK_SUCCESS) return HFRK_INVALID_CONFIG;
         plan->grid = (int)g;
         return HFRK_SUCCESS;
@@ -897,9 +901,9 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
         if (fits && band_rows >= 48 && k != 2048 && k < 16384 && make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
-    if (k >= 16384 && make_split_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
-    if (make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
-    if (make_split_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
+    if (k >= 16384 && make_split_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
+    if (make_whole_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
+    if (make_split_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     const double weight_mb = (double)n * k / 1.0e6;
     // 2 x 4 also on k = 16384 from 8192 rows on (up to 48 activation rows: 8192 x 16384 25.3 against 27+ us at 32 and 27.8
