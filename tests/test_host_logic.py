@@ -233,6 +233,46 @@ def test_plan_covers_every_unit_once_and_contributor_formula(m, n, k):
             assert p in (first_panel, last_panel) or (ub(g) <= lo and hi <= ub(g + 1))
 
 
+def test_planner_on_random_shapes_gives_plans_the_launcher_accepts_and_that_cover_the_work():
+    """The planner's rules are many and were read off sweeps of particular shapes: on 400 seeded random shapes (row counts
+    1..64, weights of 16..60000 rows including ragged ones, k up to 32768 in steps of 256, a third of them in the packed
+    load format) whatever it answers must pass the
+    launcher's own check (hfrk_plan_table_set runs it) and, replayed on the host, multiply every unit of work exactly once."""
+    import random
+    from hf_rocm_kernels import plan_table
+    rng = random.Random(20250)
+    lib = _capi.load()
+    kinds = set()
+    plan_table.clear()
+    try:
+        for _ in range(400):
+            m = rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 20, 24, 25, 28, 32, 33, 40, 48, 49, 64])
+            n = rng.choice([rng.randrange(16, 60000), 64 * rng.randrange(1, 900), 128 * rng.randrange(1, 450), 4 * rng.randrange(4, 15000)])
+            k = 256 * rng.choice([rng.randrange(1, 129), rng.choice([4, 8, 12, 16, 20, 32, 56, 64, 112])])
+            p = _capi.GemmPlan()
+            packed = rng.randrange(3) == 0  # the planner's answer for weights in the packed load format (empty table: its rules)
+            status = lib.hfrk_plan_table_get(m, n, k, int(packed), ctypes.byref(p))
+            assert status == _capi.SUCCESS, (m, n, k, packed, _capi.status_string(status))
+            assert lib.hfrk_plan_table_set(m, n, k, int(packed), ctypes.byref(p)) == _capi.SUCCESS, (m, n, k, packed, p.as_dict())
+            plan_table.clear()
+            assert not packed or p.wn != -2  # bands of any 4-row height do not exist in 16-row packed tiles
+            kinds.add(p.wn if p.wn <= 0 else 1)
+            if p.panels * p.slabs > 200000:
+                continue  # (the replay is a Python loop over units)
+            if p.wn == -2:
+                _emulate_rows(p)
+            elif p.wn == 0:
+                assert all(c == 1 for c in _emulate_stream(p)[0]), (m, n, k)
+            elif p.wn == -1:
+                r = _stream_ranges(p)
+                assert r[0][0] == 0 and r[-1][1] == p.panels * p.slabs and all(a[1] == b[0] and a[0] < a[1] for a, b in zip(r, r[1:]))
+            else:
+                assert all(c == 1 for row in _emulate(p, n, k)[0] for c in row), (m, n, k)
+    finally:
+        plan_table.clear()
+    assert kinds == {-2, -1, 0, 1}
+
+
 def test_plan_rejects_what_the_kernel_cannot_take():
     p = _capi.GemmPlan()
     lib = _capi.load()
