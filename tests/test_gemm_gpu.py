@@ -135,6 +135,28 @@ def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
     check_against_oracle(out, a, b, sa, sw, base=base)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_default_plan_on_random_shapes(seed):
+    """The planner's rules were read off sweeps of particular shapes; whatever they answer for a shape nobody swept must still
+    be the right product: seeded random row counts, weight heights (ragged ones too) and k, per-token and per-channel scales,
+    plain and accumulating, against the oracle."""
+    import random
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    rng = random.Random(7000 + seed)
+    m = rng.choice([1, 3, 4, 5, 8, 9, 13, 16, 17, 20, 24, 25, 31, 32, 33, 47, 48, 50, 64])
+    n = rng.choice([4 * rng.randrange(600, 3100), 64 * rng.randrange(40, 200), 128 * rng.randrange(20, 100), rng.randrange(2400, 12000)])
+    k = 256 * rng.choice([rng.randrange(2, 33), rng.choice([8, 12, 16, 20, 32])])
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=seed, per_token=True, per_channel=True)
+    print(f"m={m} n={n} k={k}", flush=True)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    run_ex(a, b, sa, sw, out, accumulate=False)
+    check_against_oracle(out, a, b, sa, sw)
+    base = torch.randn(m, n, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16).cuda()
+    out = base.clone()
+    run_ex(a, b, sa, sw, out, accumulate=True)
+    check_against_oracle(out, a, b, sa, sw, base=base)
+
+
 @pytest.mark.parametrize("m,n,k", [(8, 512, 2048), (16, 1040, 4096), (33, 256, 1024), (64, 6144, 4096), (5, 4096, 14336),
                                    (1, 50, 256), (13, 6144, 4096), (4, 1000, 1024),
                                    (32, 2000, 2048), (20, 1040, 1024), (25, 6144, 4096), (12, 28672, 4096),
