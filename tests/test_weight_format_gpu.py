@@ -166,6 +166,24 @@ def test_every_plan_on_a_packed_weight_equals_the_row_major_result_bit_for_bit(m
     check_against_oracle(got, a, b, sa, sw, base=base)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_default_plan_on_random_packed_weights(seed):
+    """Whatever the planner answers for a packed weight of a shape nobody swept: against the oracle, accumulating onto a base."""
+    import random
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    rng = random.Random(9100 + seed)
+    m = rng.choice([1, 4, 5, 8, 13, 16, 17, 24, 32, 33, 48, 64])
+    n = rng.choice([64 * rng.randrange(40, 200), 128 * rng.randrange(20, 100), rng.randrange(2400, 12000)])
+    k = 256 * rng.choice([rng.randrange(2, 33), rng.choice([8, 12, 16, 20, 32])])
+    print(f"m={m} n={n} k={k}", flush=True)
+    a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=seed, per_token=True, per_channel=True)
+    packed = _pack(b.t().view(torch.uint8))
+    base = torch.randn((m, n), device="cuda").to(torch.bfloat16)
+    got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    _run_fused(a, b, got, base, sa, sw, None, 0, None, packed)
+    check_against_oracle(got, a, b, sa, sw, base=base)
+
+
 @pytest.mark.parametrize("m,n,k", [(7, 1000, 1024), (40, 2048, 4096), (64, 1040, 2048)])
 def test_float16_output_and_accumulation_on_a_packed_weight(m, n, k):
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
