@@ -465,6 +465,30 @@ def test_swiglu_epilogue_matches_the_two_kernel_chain(m, n, k, per_channel, dtyp
         assert (d > 0).float().mean() < 0.02, (name, float((d > 0).float().mean()))
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_swiglu_epilogue_on_random_shapes(seed):
+    """The fused projection + SwiGLU under whatever plan the library picks for a shape nobody swept (row-split bands of output
+    columns, wave-stream, K-split above 16 rows, or the two-kernel fallback where no epilogue exists): against the oracle."""
+    import random
+    from hf_rocm_kernels import skinny_gemm_swiglu
+    from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
+    rng = random.Random(5300 + seed)
+    m = rng.choice([1, 2, 4, 5, 8, 12, 16, 17, 32, 40, 64])
+    n = 32 * rng.choice([rng.randrange(16, 400), rng.randrange(100, 900)])
+    k = 256 * rng.choice([rng.randrange(2, 33), 8, 16, 16, 32])
+    print(f"m={m} n={n} k={k}", flush=True)
+    a, w, sa, sw = generate_llama_gemm_data(m, n, k, seed=seed, per_token=(m > 4), per_channel=bool(seed & 1), weight_std=0.05)
+    out_scale = torch.tensor([8.0 / 448], dtype=torch.float32).cuda()
+    fused = skinny_gemm_swiglu(a, w, sa, sw, out_scale)
+    assert fused.dtype == torch.float8_e4m3fn and fused.shape == (m, n // 2)
+    ref, tol = _swiglu_oracle(a, w, sa, sw, out_scale, torch.bfloat16)
+    f = fused.cpu().float()
+    assert not f.isnan().any()
+    d = (f - ref.float()).abs()
+    assert (d <= tol).all(), float((d / tol).max())
+    assert (d > 0).float().mean() < 0.02, float((d > 0).float().mean())
+
+
 def test_swiglu_epilogue_limits_and_fallback():
     from hf_rocm_kernels import _capi, skinny_gemm_swiglu
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
