@@ -790,11 +790,15 @@ static int fill_workgroup_plan(int m, int n, int k, int wn, int ch, hfrk_gemm_pl
 //   / 49.8, 16384 rows on 256 46.8 / 48.5 against 47.4 / 52.2 (with one chunk per slab it is 6-7 % behind there).
 static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = false) {
     const int mt = (m + 15) / 16;
-    const int heights[3] = {256, 128, 64};
-    for (int hi = 0; hi < 3; ++hi) {
+    const int heights[4] = {256, 128, 64, 32};
+    for (int hi = 0; hi < 4; ++hi) {
         const int h = heights[hi];
         if (n % h != 0) continue;
         const long panels = n / h;
+        // 32-row panels (2 row waves x 4 K waves), one each on 224..256 workgroups: short k that no K-split window covers, up to
+        // 48 rows (8192 x 3072 9.7 / 10.1 us at 33 / 48 rows against 11.2 / 11.4, 7168 x 5120 12.5 / 13.1 against 13.5 / 14.0; at
+        // 64 rows level or 9 % behind, at k = 8192 18-27 % behind, at k = 2048 / 4096 7-24 % behind the K-split kernel)
+        if (h == 32 && (panels > kNumCU || k > 5120 || k == 2048 || k == 4096 || m > 48)) continue;
         long g_try[2] = {0, 0};  // several panels each on 224..256 workgroups; one panel each on fewer
         if (k <= 8192)
             for (long g = kNumCU; g >= 7 * kNumCU / 8 && !g_try[0]; g -= 8)
@@ -815,7 +819,7 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool
         for (int gi = 0; gi < 2; ++gi) {
             const long g = g_try[gi];
             if (g == 0) continue;
-            const int wn = h == 64 ? 4 : 8, wk = kGemmWaves / wn, rt = h == 256 ? 2 : 1;
+            const int wn = h == 32 ? 2 : h == 64 ? 4 : 8, wk = kGemmWaves / wn, rt = h == 256 ? 2 : 1;
             // two chunks per slab on short k with 8 row waves (28672 x 4096 at 64 rows: 25.4 against 26.5 us), else one
             int ch = ((wn == 8 && rt == 1 && k <= 5120 && k % 512 == 0) || (wn == 4 && k > 14336)) ? 2 : 1;
             if (lds_bytes_for(mt, wk, ch, rt) > kLdsLimit) ch = 1;

@@ -110,7 +110,8 @@ def test_default_plan_matches_oracle(m, n, k):
                                    (33, 13312, 14336), (48, 24576, 16384), (64, 20480, 3072), (40, 16384, 16384),
                                    (48, 13312, 16384), (32, 6144, 16384), (64, 8192, 16384), (17, 6144, 14336),
                                    (20, 14336, 5120), (24, 16384, 14336), (18, 13312, 8192),
-                                   (8, 5120, 8192), (4, 5120, 8192), (16, 5120, 5120), (7, 7168, 14336), (5, 11264, 5120)])
+                                   (8, 5120, 8192), (4, 5120, 8192), (16, 5120, 5120), (7, 7168, 14336), (5, 11264, 5120),
+                                   (48, 8192, 3072), (33, 7168, 5120)])
 def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
     """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), ragged bands of
     20..44 rows (two weight tiles per chunk from 5 rows on), the 17..32 row
@@ -124,7 +125,7 @@ def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
         assert p.wn == -2
     else:
         panels = n // (16 * p.wn)
-        assert p.wn in (4, 8, 16) and (panels % p.grid == 0 or p.grid % panels == 0), p.as_dict()   # whole panels, or whole fractions
+        assert p.wn in (2, 4, 8, 16) and (panels % p.grid == 0 or p.grid % panels == 0), p.as_dict()   # whole panels, or whole fractions
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=m + n + k, per_token=True, per_channel=True)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     run_ex(a, b, sa, sw, out, accumulate=False)

@@ -359,6 +359,9 @@ def test_workgroup_plans_on_whole_and_split_panels():
     assert plan(32, 6144, 16384)[1:6] == (8, 1, 1, 192, 48)
     assert plan(32, 6144, 14336)[1:6] == (8, 1, 1, 192, 48)
     assert plan(48, 8192, 16384)[1:3] == (2, 4) and plan(64, 8192, 16384)[1:6] == (8, 1, 1, 256, 64)
+    # 32-row panels (2 row waves x 4 K waves), one each, on short k that no K-split window covers, up to 48 rows
+    assert plan(48, 8192, 3072)[1:6] == (2, 4, 1, 256, 256) and plan(33, 7168, 5120)[1:6] == (2, 4, 1, 224, 224)
+    assert plan(64, 8192, 3072)[1:3] == (4, 2) and plan(48, 8192, 8192)[1:3] == (4, 2) and plan(48, 8192, 4096)[1] == -1
     # 17..24 rows: whole 64-row panels come before the row-split kernel from 12288 weight rows on
     assert plan(24, 13312, 8192)[1:6] == (4, 2, 1, 208, 208) and plan(20, 16384, 14336)[1:6] == (4, 2, 1, 256, 256)
     assert plan(24, 10240, 8192)[1] == -2 and plan(19, 16384, 2048)[1] == -2 and plan(24, 16384, 16384)[1] == -2
