@@ -795,8 +795,9 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool
         const int h = heights[hi];
         if (n % h != 0) continue;
         const long panels = n / h;
-        // 32-row panels (2 row waves x 4 K waves), one each on 224..256 workgroups: short k that no K-split window covers, up to
-        // 48 rows (8192 x 3072 9.7 / 10.1 us at 33 / 48 rows against 11.2 / 11.4, 7168 x 5120 12.5 / 13.1 against 13.5 / 14.0; at
+        // 32-row panels (2 row waves x 4 K waves), one each on 160..256 workgroups: short k that no K-split window covers, up to
+        // 48 rows (8192 x 3072 9.7 / 10.1 us at 33 / 48 rows against 11.2 / 11.4, 7168 x 5120 12.5 / 13.1 against 13.5 / 14.0,
+        // 6144 x 3072 on 192 workgroups 9.2 / 9.6 against 10.6 / 10.9, 5120 x 5120 on 160 11.8 / 12.4 against 12.9 / 13.1; at
         // 64 rows level or 9 % behind, at k = 8192 18-27 % behind, at k = 2048 / 4096 7-24 % behind the K-split kernel)
         if (h == 32 && (panels > kNumCU || k > 5120 || k == 2048 || k == 4096 || m > 48)) continue;
         long g_try[2] = {0, 0};  // several panels each on 224..256 workgroups; one panel each on fewer
@@ -814,6 +815,7 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool
             // (packed weights, 24576 x 8192: 42.0 / 41.9 / 45.2 us at 20 / 32 / 64 rows against 36.4 / 36.6 / 43.2 for the rules
             // below -- a panel is 1 MB of contiguous bytes there; k = 3072, 5120 and 16384 gain 11-24 % in both layouts)
             if (h == 128 && packed && k == 8192) one_each = false;
+            if (h == 32) one_each = panels >= 160;
             if (one_each) g_try[1] = panels;
         }
         for (int gi = 0; gi < 2; ++gi) {

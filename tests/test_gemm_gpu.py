@@ -111,7 +111,7 @@ def test_default_plan_matches_oracle(m, n, k):
                                    (48, 13312, 16384), (32, 6144, 16384), (64, 8192, 16384), (17, 6144, 14336),
                                    (20, 14336, 5120), (24, 16384, 14336), (18, 13312, 8192),
                                    (8, 5120, 8192), (4, 5120, 8192), (16, 5120, 5120), (7, 7168, 14336), (5, 11264, 5120),
-                                   (48, 8192, 3072), (33, 7168, 5120)])
+                                   (48, 8192, 3072), (33, 7168, 5120), (40, 5120, 5120)])
 def test_default_plan_on_shapes_with_rules_of_their_own(m, n, k):
     """Weights whose bands come to 512 KB (two weight tiles per chunk, or 256 workgroups instead of 224), ragged bands of
     20..44 rows (two weight tiles per chunk from 5 rows on), the 17..32 row

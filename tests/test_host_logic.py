@@ -361,6 +361,7 @@ def test_workgroup_plans_on_whole_and_split_panels():
     assert plan(48, 8192, 16384)[1:3] == (2, 4) and plan(64, 8192, 16384)[1:6] == (8, 1, 1, 256, 64)
     # 32-row panels (2 row waves x 4 K waves), one each, on short k that no K-split window covers, up to 48 rows
     assert plan(48, 8192, 3072)[1:6] == (2, 4, 1, 256, 256) and plan(33, 7168, 5120)[1:6] == (2, 4, 1, 224, 224)
+    assert plan(48, 6144, 3072)[1:6] == (2, 4, 1, 192, 192) and plan(40, 5120, 5120)[1:6] == (2, 4, 1, 160, 160)
     assert plan(64, 8192, 3072)[1:3] == (4, 2) and plan(48, 8192, 8192)[1:3] == (4, 2) and plan(48, 8192, 4096)[1] == -1
     # 17..24 rows: whole 64-row panels come before the row-split kernel from 12288 weight rows on
     assert plan(24, 13312, 8192)[1:6] == (4, 2, 1, 208, 208) and plan(20, 16384, 14336)[1:6] == (4, 2, 1, 256, 256)
