@@ -936,7 +936,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
         if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
         if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
         if (p->m_tiles != 1 || p->panels != (n + 3) / 4 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
-        if (p->grid < 1 || p->grid > kMaxGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
+        if (p->grid < 1 || p->grid > kMaxStreamGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
         if (p->lds_bytes != rows_lds_bytes(p->wk, p->ch)) return HFRK_INVALID_CONFIG;
         // a band's chunk indices stay far below 2^32 / slabs (the kernel divides by multiplying with a reciprocal)
         if (((long)p->panels / p->grid / 4 + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;
@@ -961,7 +961,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
         const int rows = swiglu ? 16 : 16 * p->wk;  // with the SwiGLU epilogue n counts output columns: one gate + one up tile
         if (p->panels != (n + rows - 1) / rows || p->slabs != (k + 255) / 256 || p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
         const long chunks = (long)p->panels * p->slabs;
-        if (p->grid < 1 || p->grid > kMaxGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
+        if (p->grid < 1 || p->grid > kMaxStreamGrid || p->grid > chunks) return HFRK_INVALID_CONFIG;
         if (chunks * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's chunk arithmetic is 32-bit
         if (p->lds_bytes != stream_lds_bytes(p->ch, p->wk)) return HFRK_INVALID_CONFIG;
         return HFRK_SUCCESS;
@@ -972,12 +972,14 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
     const int rt = p->wn * p->wk / kGemmWaves;
     if (p->wn < 1 || p->wn * p->wk != rt * kGemmWaves || (rt != 1 && rt != 2)) return HFRK_INVALID_CONFIG;
     if (p->ch != 1 && p->ch != 2) return HFRK_INVALID_CONFIG;
-    if (rt == 2 && (p->ch != 1 || p->grid > kMaxGrid / 2)) return HFRK_INVALID_CONFIG;  // registers; workspace slots are twice as large
+    if (rt == 2 && p->ch != 1) return HFRK_INVALID_CONFIG;  // registers
     const int ks = 256 * p->wk * p->ch, bn = 16 * p->wn;
     if (k % ks != 0 || p->slabs != k / ks || p->panels != (n + bn - 1) / bn) return HFRK_INVALID_CONFIG;
     if (p->panels > kMaxPanels) return HFRK_INVALID_CONFIG;
     const long units = (long)p->panels * p->slabs;
-    if (p->grid < 1 || p->grid > kMaxGrid || p->grid > units) return HFRK_INVALID_CONFIG;
+    // One workgroup per compute unit at most: with more, workgroups of up to 160 KB of LDS run in two rounds over shared
+    // partial-sum slots and arrival counters, a regime no test of this kernel covers (see kMaxStreamGrid).
+    if (p->grid < 1 || p->grid > kNumCU || p->grid > units) return HFRK_INVALID_CONFIG;
     if (units * (p->grid + 1) >= (1L << 31)) return HFRK_BAD_SHAPE;  // the kernel's unit arithmetic is 32-bit
     if (p->lds_bytes != lds_bytes_for(p->m_tiles, p->wk, p->ch, rt) || p->lds_bytes > kLdsLimit) return HFRK_INVALID_CONFIG;
     return HFRK_SUCCESS;

@@ -11,7 +11,13 @@ constexpr int kTileBytes = 4096;       // 16 rows x 256 B: one K chunk of one 16
 constexpr int kLdsLimit = 160 * 1024;  // LDS per CU on gfx950
 constexpr int kMaxPanels = 1 << 20;    // arrival counters (one per row panel / row tile)
 constexpr int kMaxDevices = 64;     // devices this library keeps per-device state for
-constexpr int kMaxGrid = 4 * kNumCU;   // persistent workgroups: up to 4 per CU when LDS and registers allow
+constexpr int kMaxGrid = 4 * kNumCU;   // what the workspace is sized for
+// Largest grid a plan may ask for.  The row-split and wave-stream kernels take up to two workgroups per compute unit (the
+// planner itself uses that for short bands at up to 4 rows, and forced plans of that size are part of the GPU tests); the
+// K-split and workgroup kernels take one.  Larger grids were accepted once; a tuner sweep that forced them on 2048-row
+// weights ended in a GPU fault whose cause was never found, no test covers them, and no measurement ever favoured them,
+// so the launcher refuses them.
+constexpr int kMaxStreamGrid = 2 * kNumCU;
 constexpr size_t kWsFloats = (size_t)2 * kMaxGrid * kGemmWaves * 4 * 256;  // 2 slots x grid x up to 32 KB of fp32 partials
 
 struct GemmArgs {
