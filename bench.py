@@ -22,7 +22,10 @@ Other workloads, same method, for the remaining configurations:
   pack        the step before the path: the four Llama-3-8B weights packed into the load format from float8_e4m3fn,
               packed from float8_e4m3fnuz (re-encoded on the way) and unpacked again: 12 launches per step, 2*N*K
               bytes each (`hf_rocm_kernels.utils.weight_format`)
-  floor       what bounds a launch from below, measured with the library's probe kernels: an empty kernel with the GEMM's
+  elementwise the two kernels either side of the GEMM at the sizes the reference publishes times for (its
+              benchmarks/residual_rms/vs_reference.py:50-61, benchmarks/swiglu/vs_reference.py:43-55): residual RMSNorm -> fp8 on
+              16384 columns and SwiGLU -> fp8 on 6656, rows 1, 8, 64, 256, 2048 each, float16 in; `cases` holds microseconds and GB/s
+  floor       what bounds a launch from below, measured with probe kernels (a bench-only library): an empty kernel with the GEMM's
               launch geometry as a graph node, the row-split GEMM's weight requests alone (no activations, no LDS, no matrix
               instructions, no output) for each of the eight Llama-3 8B / 70B weights, and the same on a 1.9 GB weight for
               the sustained read rate; `cases` holds the table
@@ -37,7 +40,8 @@ roofline    = the same bytes over the same HIP-event time, against 8 TB/s of HBM
 cpu_baseline= the oracle's torch path (dequantise -> fp32 matmul -> scale -> bf16) on the host cores, same shapes
 traffic     = HBM bytes per launch read back from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE runs of this
               script with `--copy-calibration`, which appends a plain 256 MiB device copy whose counter reading
-              fixes the scale); the figure is a constant below because a benchmark cannot profile itself
+              fixes the scale).  A benchmark cannot profile itself: the figure is a constant recorded from those runs
+              (`roofline.traffic_source` names the summary under profiles/ it comes from), null for workloads without one
 
 Before the timed steps the graphs are replayed for at least 0.3 s (`config.preroll_ms`), so that a short run and a long
 one see the same clocks.  After them every (shape, M) case is timed on its own, outside the timed region (`cases`:
@@ -59,6 +63,8 @@ HBM_PEAK_GBPS = 8000.0
 # Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
 # runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0094 x the algorithmic bytes.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55216472}
+MEASURED_TRAFFIC_SOURCE = {"llama3-8b": "recorded constant, not measured by this run: profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt "
+                                        "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy)"}
 CALIBRATION_COPY_BYTES = 256 << 20
 
 WORKLOADS = {
@@ -494,6 +500,79 @@ def run_pack_workload(torch, args):
     return result
 
 
+# ---- the two element-wise kernels at the reference's sizes ---------------------------------------------------------------
+
+def run_elementwise_workload(torch, args):
+    """Residual RMSNorm -> fp8 (16384 columns) and SwiGLU -> fp8 (6656 columns) at 1, 8, 64, 256, 2048 rows, float16 in: the
+    sizes the reference publishes times for.  A step is the ten launches; every case is also timed on its own."""
+    from hf_rocm_kernels import residual_rms, swiglu
+    from hf_rocm_kernels.operators.residual_rms import generate_residual_rms_data
+    from hf_rocm_kernels.operators.swiglu import generate_swiglu_data
+    rows_list, rms_cols, swiglu_cols = [1, 8, 64, 256, 2048], 16384, 6656
+    # microseconds the reference's scripts record for its vectorised kernels (on MI300X)
+    ref_us = {"residual_rms": dict(zip(rows_list, [4.66, 4.75, 5.67, 9.47, 65.8])),
+              "swiglu": dict(zip(rows_list, [2.09, 2.15, 2.28, 3.81, 19.9]))}
+    calls = []
+    for rows in rows_list:
+        x, r, w, eps, scale, nb = generate_residual_rms_data(rows, rms_cols, 0, dtype=torch.float8_e4m3fn, seed=0)
+        out = torch.empty((rows, rms_cols), dtype=torch.float8_e4m3fn, device="cuda")
+        calls.append(("residual_rms", rows, rms_cols, rms_bytes(rows, rms_cols),
+                      (lambda x=x, r=r, w=w, eps=eps, scale=scale, nb=nb: residual_rms(x, r, w, eps, scale_tensor=scale, next_buffer=nb))))
+        gu, sc, nb2 = generate_swiglu_data(rows, swiglu_cols, 0, seed=0)
+        calls.append(("swiglu", rows, swiglu_cols, swiglu_bytes(rows, swiglu_cols), (lambda gu=gu, sc=sc, nb2=nb2: swiglu(gu, sc, nb2))))
+    stream = torch.cuda.Stream()
+
+    def graph_of(fns, repeat=1):
+        with torch.cuda.stream(stream):
+            for f in fns:
+                f()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for _ in range(repeat):
+                for f in fns:
+                    f()
+        return g
+
+    step = graph_of([c[4] for c in calls])
+    preroll_ms = preroll(torch, [step])
+    for _ in range(args.warmup):
+        step.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    step_bytes = sum(c[3] for c in calls)
+    gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    cases = []
+    for name, rows, cols, nbytes, fn in calls:
+        g = graph_of([fn], repeat=32)
+        us, std = time_graph(torch, g, 32, 40)
+        cases.append({"kernel": name, "rows": rows, "cols": cols, "us": round(us, 3), "us_std": round(std, 3), "bytes": nbytes,
+                      "gbps": round(nbytes / us / 1e3, 1), "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                      "reference_us_mi300x": ref_us[name][rows]})
+        del g
+    big = max(cases, key=lambda c: c["gbps"])
+    return {
+        "metric": "residual RMSNorm -> fp8 (16384 columns) and SwiGLU -> fp8 (6656 columns) at the reference's row counts, achieved HBM GB/s",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "residual_rms (fp16 in, fp8 out, 16384 columns) and swiglu (fp16 in, fp8 out, 6656 columns) at rows 1, 8, 64, "
+                               "256, 2048: 10 launches per step; the inputs of a case stay cache-resident between replays, as in the reference's scripts",
+                   "calls_per_step": len(calls), "bytes_per_step": step_bytes, "timing": "HIP graph replay, HIP events",
+                   "preroll_ms": round(preroll_ms, 1)},
+        "roofline": {"bound": "hbm", "achieved": big["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": big["frac_of_peak"],
+                     "traffic": None, "kernel": "hfrk::%s_vec_kernel at %d rows (the largest case; the small ones are launch-bound)" % (big["kernel"], big["rows"]),
+                     "bytes_per_launch": big["bytes"], "us_per_launch": big["us"]},
+        "cases": cases,
+    }
+
+
 def preroll(torch, graphs, seconds=0.3):
     """Replay the graphs until `seconds` of wall time have passed; returns the milliseconds it took."""
     t0 = time.perf_counter()
@@ -508,10 +587,21 @@ def preroll(torch, graphs, seconds=0.3):
 
 
 def run_floor_workload(torch, args):
-    """Launch floor, weight-stream-only time per shape and sustained read rate, from the library's probe kernels."""
-    from hf_rocm_kernels import _capi
-    lib = _capi.load()
-    _capi.check(lib.hfrk_init(), "hfrk_init")
+    """Launch floor, weight-stream-only time per shape and sustained read rate, from the probe kernels of
+    hf_rocm_kernels/benchmarks/libhfrk_bench_probes.so (built by hf-rocm-kernels_amd/build.py from bench_probes/probe.hip)."""
+    import ctypes
+    path = os.path.join(ROOT, "hf-rocm-kernels_amd", "hf_rocm_kernels", "benchmarks", "libhfrk_bench_probes.so")
+    if not os.path.exists(path):
+        sys.exit(path + " is missing: build it with `python hf-rocm-kernels_amd/build.py`")
+    lib = ctypes.CDLL(path)
+    lib.probe_empty_launch.restype = ctypes.c_int
+    lib.probe_empty_launch.argtypes = [ctypes.c_void_p]
+    lib.probe_weight_stream.restype = ctypes.c_int
+    lib.probe_weight_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+
+    def check(status, what):
+        if status != 0:
+            raise RuntimeError("%s failed with hipError_t %d" % (what, status))
     arena = torch.randint(0, 120, (3 << 30,), dtype=torch.uint8, device="cuda")
     sink = torch.zeros(16, dtype=torch.int32, device="cuda")
     stream = torch.cuda.Stream()
@@ -531,13 +621,13 @@ def run_floor_workload(torch, args):
 
     def probe(offset, n, k, grid=256):
         def call():
-            _capi.check(lib.hfrk_probe_weight_stream(arena.data_ptr() + offset, sink.data_ptr(), n, k, k, grid, raw()), "hfrk_probe_weight_stream")
+            check(lib.probe_weight_stream(arena.data_ptr() + offset, sink.data_ptr(), n, k, k, grid, raw()), "probe_weight_stream")
         return call
 
     big_n, big_k = 229376, 8192  # 1.88 GB in one launch
     big = graph_of([probe(0, big_n, big_k)])
     pre_ms = preroll(torch, [big])
-    empty = graph_of([lambda: _capi.check(lib.hfrk_probe_empty_launch(raw()), "hfrk_probe_empty_launch")] * 64)
+    empty = graph_of([lambda: check(lib.probe_empty_launch(raw()), "probe_empty_launch")] * 64)
     empty_us, _ = time_graph(torch, empty, 64, 40)
     big_us, _ = time_graph(torch, big, 1, 20)
     sustained = big_n * big_k / big_us / 1e3
@@ -559,8 +649,8 @@ def run_floor_workload(torch, args):
         "value": round(sustained, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(big_us / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
-        "config": {"workload": "probe kernels of libhfrk_gfx950.so: hfrk_probe_empty_launch (256 x 512 threads, 64 KB LDS) x 64 in a graph; "
-                               "hfrk_probe_weight_stream on a %d x %d weight (%.2f GB) and on the eight Llama-3 8B / 70B weights, "
+        "config": {"workload": "probe kernels of libhfrk_bench_probes.so: probe_empty_launch (256 x 512 threads, 64 KB LDS) x 64 in a graph; "
+                               "probe_weight_stream on a %d x %d weight (%.2f GB) and on the eight Llama-3 8B / 70B weights, "
                                "one graph node per weight copy (HBM-cold) and 32 nodes on one copy (cache-hot)" % (big_n, big_k, big_n * big_k / 1e9),
                    "preroll_ms": round(pre_ms, 1), "timing": "HIP graph replay, HIP events, median of 40"},
         "roofline": {"bound": "hbm", "achieved": round(sustained, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -576,7 +666,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=140)
     ap.add_argument("--warmup", type=int, default=28)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "mlp-rms", "pack", "floor"], default="llama3-8b")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["mlp", "mlp-fused", "mlp-rms", "pack", "floor", "elementwise"], default="llama3-8b")
     ap.add_argument("--detail", action="store_true", help="kept for older command lines: the per-case table is on by default")
     ap.add_argument("--no-cases", action="store_true", help="skip the per-case table after the timed steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -601,6 +691,9 @@ def main():
         return
     if args.workload == "floor":
         print(json.dumps(run_floor_workload(torch, args)))
+        return
+    if args.workload == "elementwise":
+        print(json.dumps(run_elementwise_workload(torch, args)))
         return
     if args.ms:
         rows = [int(x) for x in args.ms.split(",")]
@@ -681,6 +774,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": None if args.packed else MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+                     "traffic_source": None if args.packed else MEASURED_TRAFFIC_SOURCE.get(args.workload),
                      "kernel": kernel,
                      "bytes_per_launch": round(step_bytes / calls), "us_per_launch": round(ms_per_step * 1e3 / calls, 3)},
     }

@@ -1,7 +1,13 @@
-// Measurement probes: what a launch costs before it does anything, and what the GEMM's own weight requests cost when
-// nothing is computed.  They give the floor the skinny-GEMM kernels are measured against (launch + first-byte latency +
-// bytes / sustained bandwidth), per weight shape.  No counterpart in the reference, which publishes timings only
-// (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:45-88).
+// Measurement probes, built into a library of their own (libhfrk_bench_probes.so) that only `bench.py --workload floor`
+// loads: they are not part of libhfrk_gfx950.so or its header.  What a launch costs before it does anything, and what the
+// GEMM's own weight requests cost when nothing is computed: the floor the skinny-GEMM kernels are measured against (launch +
+// first-byte latency + bytes / sustained bandwidth), per weight shape.  No counterpart in the reference, which publishes
+// timings only (hf_rocm_kernels/operators/skinny_gemm/wrapped.py:45-88).
+//   probe_empty_launch    a kernel with the GEMM's launch geometry (256 workgroups x 512 threads, 64 KB of LDS) that does
+//                         nothing: what a launch (or a graph node) costs before its first instruction.
+//   probe_weight_stream   the row-split GEMM's weight requests for B [n, k] (row stride b_stride) on `grid` workgroups and
+//                         nothing else.  `sink` is 4 writable bytes that are never written in practice.  k >= 512, k % 256 == 0.
+// Both return 0 or a hipError_t.
 #include "skinny_gemm_args.h"
 
 namespace hfrk {
@@ -73,19 +79,18 @@ __global__ void __launch_bounds__(kGemmThreads) probe_weight_stream_kernel(const
 
 extern "C" {
 
-int hfrk_probe_empty_launch(void* stream) {
+int probe_empty_launch(void* stream) {
     static int* sink = nullptr;  // never dereferenced by the kernel
     hipLaunchKernelGGL(hfrk::probe_empty_kernel, dim3(hfrk::kNumCU), dim3(hfrk::kGemmThreads), 64 * 1024, static_cast<hipStream_t>(stream), sink);
-    HFRK_HIP_TRY(hipGetLastError());
-    return HFRK_SUCCESS;
+    return (int)hipGetLastError();
 }
 
-int hfrk_probe_weight_stream(const void* B, void* sink, int n, int k, int b_stride, int grid, void* stream) {
+int probe_weight_stream(const void* B, void* sink, int n, int k, int b_stride, int grid, void* stream) {
     if (!B || !sink || n < 1 || k < 512 || k % 256 != 0 || b_stride < k || (b_stride & 15) || (reinterpret_cast<uintptr_t>(B) & 15))
-        return HFRK_BAD_SHAPE;
-    if (((long)n + 128) * b_stride + k >= (1L << 31)) return HFRK_BAD_SHAPE;
+        return (int)hipErrorInvalidValue;
+    if (((long)n + 128) * b_stride + k >= (1L << 31)) return (int)hipErrorInvalidValue;
     const int units = (n + 3) / 4;
-    if (grid < 1 || grid > hfrk::kMaxGrid || grid > units) return HFRK_INVALID_CONFIG;
+    if (grid < 1 || grid > hfrk::kMaxStreamGrid || grid > units) return (int)hipErrorInvalidValue;
     hfrk::GemmArgs args = {};
     args.B = static_cast<const uint8_t*>(B);
     args.D = sink;
@@ -105,8 +110,7 @@ int hfrk_probe_weight_stream(const void* B, void* sink, int n, int k, int b_stri
     geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
     args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)args.slabs - 1) / (uint64_t)args.slabs);
     hipLaunchKernelGGL(hfrk::probe_weight_stream_kernel, dim3(grid), dim3(hfrk::kGemmThreads), 0, static_cast<hipStream_t>(stream), args);
-    HFRK_HIP_TRY(hipGetLastError());
-    return HFRK_SUCCESS;
+    return (int)hipGetLastError();
 }
 
 }  // extern "C"

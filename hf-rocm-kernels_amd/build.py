@@ -2,6 +2,8 @@
 
   hf_rocm_kernels/libhfrk_gfx950.so   HIP kernels + C ABI (include/hfrk_gfx950.h); depends on the HIP runtime only
   hf_rocm_kernels/_HFRK_C.abi3.so     torch.ops._HFRK_C registration, a thin caller of the C ABI
+  hf_rocm_kernels/benchmarks/libhfrk_bench_probes.so   measurement probes for `bench.py --workload floor` (bench_probes/probe.hip);
+                                      not part of the product library
 
 Plain hipcc / g++ command lines: no cmake, no hipify, no CUDA-compat headers (the reference's CMakeLists.txt,
 cmake/utils.cmake and cmake/hipify.py have no counterpart here).  hipcc cross-compiles, so no GPU is needed.
@@ -24,7 +26,9 @@ INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["hfrk_common.hip", "skinny_gemm.hip", "skinny_gemm_stream.hip", "skinny_gemm_rows.hip", "skinny_gemm_ksplit.hip", "residual_rms.hip", "swiglu.hip",
-               "dynamic_quant.hip", "pack_weight.hip", "plan_table_file.hip", "probe.hip"]
+               "dynamic_quant.hip", "pack_weight.hip", "plan_table_file.hip"]
+PROBE_SOURCE = os.path.join(HERE, "bench_probes", "probe.hip")
+PROBE_LIB = os.path.join(PKG, "benchmarks", "libhfrk_bench_probes.so")
 LIB_NAME = "libhfrk_gfx950.so"
 EXT_NAME = "_HFRK_C.abi3.so"
 
@@ -75,6 +79,12 @@ def _compile_torch_bindings():
     return obj
 
 
+def _build_probes():
+    hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
+    _run([hipcc] + HIPCC_FLAGS + ["-shared", PROBE_SOURCE, "-o", PROBE_LIB, "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    return PROBE_LIB
+
+
 def _link_library(objs):
     hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path()] + objs +
@@ -99,7 +109,9 @@ def build_all(with_torch=True):
     with ThreadPoolExecutor(max_workers=6) as pool:
         hip_jobs = [pool.submit(_compile_hip, s) for s in HIP_SOURCES]
         ext_job = pool.submit(_compile_torch_bindings) if with_torch else None
+        probe_job = pool.submit(_build_probes)
         objs = [j.result() for j in hip_jobs]
+        probe_job.result()
         _link_library(objs)
         if ext_job is not None:
             _link_torch_extension(ext_job.result())

@@ -272,13 +272,11 @@ int64_t gemm_fused_common(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, 
     TORCH_CHECK(A.dim() == 2 && A.is_contiguous(), "A must be a contiguous [m, k] tensor");
     check_fp8(A, "A");
     check_fp8(B, "B");
-    bool scales_in_buffer = false;  // a buffer of pack_weight_scaled: its per-channel scales apply when scale_b is None
     if (packed) {
         TORCH_CHECK(n >= 1 && n < (int64_t(1) << 30) && A.size(1) < (int64_t(1) << 30), "n and k must fit 30 bits");
         const size_t plain = hfrk_packed_weight_bytes((int)n, (int)A.size(1)), scaled = hfrk_packed_weight_bytes_scaled((int)n, (int)A.size(1));
         TORCH_CHECK(B.is_contiguous() && B.numel() > 0 && ((size_t)B.numel() == plain || (size_t)B.numel() == scaled),
                     "B must be the packed buffer of a [n, k] weight (pack_weight, pack_weight_scaled) with k = A.size(1)");
-        scales_in_buffer = (size_t)B.numel() == scaled;
     } else {
         TORCH_CHECK(B.dim() == 2 && B.size(0) == A.size(1) && B.stride(0) == 1, "B must be [k, n] with unit stride along k");
     }
@@ -288,7 +286,9 @@ int64_t gemm_fused_common(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, 
     TORCH_CHECK(scale_a.scalar_type() == at::kFloat && scale_a.is_contiguous() && (scale_a.numel() == 1 || scale_a.numel() == m),
                 "scale_a must be float32 with 1 or m elements");
     check_same_device(A, scale_a, "scale_a");
-    const float* scale_b_ptr = nullptr;  // None = 1
+    // None = 1, in either weight layout: the scales a pack_weight_scaled buffer carries apply only when the caller passes
+    // them (PackedWeight.scales is a view of that part of the buffer), so one call means one thing whatever the layout.
+    const float* scale_b_ptr = nullptr;
     int sb_stride = 0;
     if (scale_b.has_value()) {
         TORCH_CHECK(scale_b->scalar_type() == at::kFloat && scale_b->is_contiguous() && (scale_b->numel() == 1 || scale_b->numel() == n),
@@ -296,8 +296,6 @@ int64_t gemm_fused_common(at::Tensor& A, at::Tensor& B, bool packed, int64_t n, 
         check_same_device(A, *scale_b, "scale_b");
         scale_b_ptr = scale_b->data_ptr<float>();
         sb_stride = scale_b->numel() == 1 ? 0 : 1;
-    } else if (scales_in_buffer) {
-        sb_stride = HFRK_SCALES_IN_PACKED_BUFFER;
     }
     int d_dtype;
     const void* base_ptr = nullptr;

@@ -87,8 +87,6 @@ SIGNATURES = {
     "hfrk_swiglu_dynamic": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
     "hfrk_quantize_fp8": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "hfrk_plan_table_load": (_i, [ctypes.c_char_p, _i, ctypes.POINTER(_i)]),
-    "hfrk_probe_empty_launch": (_i, [_p]),
-    "hfrk_probe_weight_stream": (_i, [_p, _p, _i, _i, _i, _i, _p]),
 }
 
 _lib = None

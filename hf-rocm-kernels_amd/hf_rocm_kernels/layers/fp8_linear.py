@@ -61,7 +61,11 @@ def apply_fp8_linear(
         sa = sa.reshape(-1)
     w = _weight_view(weight)
     n = w.size(1)
-    sb = None if weight_scale is None else weight_scale.reshape(-1)
+    if weight_scale is None:
+        assert isinstance(w, PackedWeight) and w.scales is not None, "a weight without scales of its own needs weight_scale"
+        sb = w.scales  # the per-channel scales stored behind the packed bytes, passed explicitly
+    else:
+        sb = weight_scale.reshape(-1)
     m = q.size(0)
     base = None
     if residual is not None:

@@ -138,8 +138,9 @@ def skinny_gemm_scaled(
     accumulate: bool = False,
 ) -> Tensor:
     """Per-token x per-output-channel variant: output[i, j] (+)= scale_a[i] * scale_b[j] * (skinny_a @ b)[i, j].
-    `scale_a` has 1 or m float32 elements, `scale_b` 1 or n; `scale_b` None takes the scales a PackedWeight carries
-    (`pack_weight(weight, scales)`).  With accumulate=False the output is overwritten.
+    `scale_a` has 1 or m float32 elements, `scale_b` 1 or n; `scale_b` None stands for `b.scales`, the scales a
+    PackedWeight carries (`pack_weight(weight, scales)`), and is an error for any other weight.  With accumulate=False
+    the output is overwritten.
     This variant has no counterpart in the reference; an omitted output is allocated as bfloat16 (the serving dtype of the
     Llama-3 checkpoints it is used with), unlike `skinny_gemm`, which keeps the reference's float16."""
     m, n = skinny_a.size(0), b.size(1)
@@ -150,11 +151,11 @@ def skinny_gemm_scaled(
     assert scale_a.numel() in (1, m) and scale_a.dtype == torch.float32, f"Expected 1 or {m} float32 in scale_a"
     if scale_b is None:
         assert isinstance(b, PackedWeight) and b.scales is not None, "scale_b may be omitted only for a PackedWeight that carries its scales"
-    else:
-        assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
+        scale_b = b.scales  # a float32 view of the packed buffer's tail: passed like any other per-channel scale
+    assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
     if isinstance(b, PackedWeight) or torch.compiler.is_compiling():
         _fused(skinny_a, b, output, output if accumulate else None, scale_a.contiguous().view(-1),
-               None if scale_b is None else scale_b.contiguous().view(-1), None, _capi.EPILOGUE_NONE, 0)
+               scale_b.contiguous().view(-1), None, _capi.EPILOGUE_NONE, 0)
         return output
     status = _skinny_gemm_scaled(skinny_a, b, output, scale_a.contiguous().view(-1), scale_b.contiguous().view(-1),
                                  accumulate)
@@ -178,7 +179,7 @@ class _ShapeOnly:
 def _scale_vectors(skinny_a: Tensor, b: Tensor, scale_a: Tensor, scale_b: Optional[Tensor]) -> Tuple[Tensor, Optional[Tensor]]:
     m, n = skinny_a.size(0), b.size(1)
     assert scale_a.numel() in (1, m) and scale_a.dtype == torch.float32, f"Expected 1 or {m} float32 in scale_a"
-    if scale_b is None:  # one combined scale in scale_a, or the scales a PackedWeight carries
+    if scale_b is None:  # one combined scale in scale_a: the weight's side of it is 1, whatever the weight's layout
         return scale_a.contiguous().view(-1), None
     assert scale_b.numel() in (1, n) and scale_b.dtype == torch.float32, f"Expected 1 or {n} float32 in scale_b"
     return scale_a.contiguous().view(-1), scale_b.contiguous().view(-1)
@@ -193,7 +194,7 @@ def skinny_gemm_add(
     output: Optional[Tensor] = None,
 ) -> Tensor:
     """output[i, j] = base[i, j] + scale_a[i] * scale_b[j] * (skinny_a @ b)[i, j], summed in fp32 and rounded once
-    (`scale_b` None = 1, or the per-channel scales of a PackedWeight that carries them).
+    (`scale_b` None = 1 in either weight layout; pass `b.scales` to apply the scales a PackedWeight carries).
     `base` has the output's shape and dtype (a residual stream, a bias broadcast beforehand); it is only read, so
     the residual add after a projection costs no extra launch and no copy."""
     m, n = skinny_a.size(0), b.size(1)

@@ -31,8 +31,9 @@ class PackedWeight:
 
     Quacks like the `[k, n]` column-major view the GEMM wrappers expect (`shape`, `size`, `stride`, `dtype`,
     `device`), so their argument checks apply unchanged; `data` is the flat float8_e4m3fn buffer.  A buffer made
-    with scales is longer by 4 bytes per padded row; `scales` is then the float32 view of its n per-channel scales,
-    which the GEMM wrappers use when they are given no `scale_b`."""
+    with scales is longer by 4 bytes per padded row; `scales` is then the float32 view of its n per-channel scales:
+    pass it as `scale_b` (`skinny_gemm_scaled` and the linear layer do so when given none).  In every other wrapper an
+    omitted `scale_b` means 1, as for a row-major weight, so that one call gives one result in both layouts."""
 
     def __init__(self, data: Tensor, n: int, k: int):
         assert data.dim() == 1 and data.is_contiguous() and data.dtype == FP8_DTYPE, "data must be a flat float8_e4m3fn tensor"

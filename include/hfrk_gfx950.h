@@ -295,16 +295,6 @@ int hfrk_swiglu_dynamic(const void* gate_up, void* output, float* scales, void* 
 int hfrk_quantize_fp8(const void* input, const float* static_scale, void* output, float* scales, int rows, int cols,
                       int io_dtype, void* stream);
 
-/* Measurement probes (no reference counterpart: the reference publishes timings only,
- * hf_rocm_kernels/operators/skinny_gemm/wrapped.py:45-88).  They give the floor a GEMM launch is measured against.
- *   hfrk_probe_empty_launch    a kernel with the GEMM's launch geometry (256 workgroups x 512 threads, 64 KB of LDS) that
- *                              does nothing: what a launch (or a graph node) costs before its first instruction.
- *   hfrk_probe_weight_stream   the row-split GEMM's weight requests for B [n, k] (row stride b_stride) on `grid` workgroups
- *                              and nothing else: no activations, no LDS, no matrix instructions, no output.  `sink` is 4
- *                              writable bytes that are never written in practice.  k >= 512, k % 256 == 0. */
-int hfrk_probe_empty_launch(void* stream);
-int hfrk_probe_weight_stream(const void* B, void* sink, int n, int k, int b_stride, int grid, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

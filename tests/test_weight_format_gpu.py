@@ -334,9 +334,11 @@ def test_packed_gemm_replays_in_a_graph():
 @pytest.mark.parametrize("m,n,k", [(8, 4096, 4096), (3, 1000, 1024), (33, 50, 256), (16, 2080, 2048)])
 def test_scales_stored_behind_the_packed_bytes(m, n, k):
     """hfrk_pack_weight_scaled: the packed bytes, then the n per-channel scales (zeros up to the padded row count), in one
-    buffer.  The GEMM told to use them (sb_stride = HFRK_SCALES_IN_PACKED_BUFFER through the C ABI, scale_b = None in
-    Python) gives the bits of the GEMM that is handed the scales separately, on the packed and on the row-major weight."""
-    from hf_rocm_kernels import skinny_gemm_add, skinny_gemm_scaled
+    buffer.  The GEMM told to use them (sb_stride = HFRK_SCALES_IN_PACKED_BUFFER through the C ABI; `pw.scales`, or no
+    scale_b to skinny_gemm_scaled, in Python) gives the bits of the GEMM that is handed the scales separately, on the packed
+    and on the row-major weight.  In every wrapper whose scale_b may be None for "1" it means 1 for this buffer too: the
+    same call gives the same numbers in both layouts."""
+    from hf_rocm_kernels import skinny_gemm, skinny_gemm_add, skinny_gemm_scaled
     from hf_rocm_kernels.operators.skinny_gemm import generate_llama_gemm_data
     from hf_rocm_kernels.utils.weight_format import PackedWeight, pack_weight, packed_weight_bytes, unpack_weight
     lib, _capi = _lib()
@@ -378,7 +380,13 @@ def test_scales_stored_behind_the_packed_bytes(m, n, k):
     check_against_oracle(skinny_gemm_scaled(a, pw, sa, None), a, b, sa, sw)
     assert torch.equal(skinny_gemm_scaled(a, pw, sa, None), skinny_gemm_scaled(a, pack_weight(w), sa, sw))
     base = torch.randn(m, n, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
-    assert torch.equal(skinny_gemm_add(a, pw, sa, None, base), skinny_gemm_add(a, pack_weight(w), sa, sw, base))
+    assert torch.equal(skinny_gemm_add(a, pw, sa, pw.scales, base), skinny_gemm_add(a, pack_weight(w), sa, sw, base))
+    # no scale_b = 1, whatever the weight carries: skinny_gemm / skinny_gemm_add on the scaled buffer equal the row-major call
+    with one_plan_for_both_layouts((m, n, k)):
+        assert torch.equal(skinny_gemm_add(a, pw, sa, None, base), skinny_gemm_add(a, b, sa, None, base))
+        one = sa[:1].contiguous()
+        zeros = lambda: torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        assert torch.equal(skinny_gemm(a, pw, one, zeros()), skinny_gemm(a, b, one, zeros()))
     # scales handed over explicitly win over the stored ones
     other = (sw * 2).contiguous()
     assert torch.equal(skinny_gemm_scaled(a, pw, sa, other), skinny_gemm_scaled(a, pack_weight(w), sa, other))
