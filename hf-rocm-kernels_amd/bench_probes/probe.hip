@@ -7,6 +7,10 @@
 //                         nothing: what a launch (or a graph node) costs before its first instruction.
 //   probe_weight_stream   the row-split GEMM's weight requests for B [n, k] (row stride b_stride) on `grid` workgroups and
 //                         nothing else.  `sink` is 4 writable bytes that are never written in practice.  k >= 512, k % 256 == 0.
+//   probe_packed_stream   the same for a weight in the packed load format (bands of whole 16-row tiles, 4 KB chunks that are
+//                         contiguous in memory).  order 0: every wave streams a contiguous run of its workgroup's chunks (what
+//                         the GEMM does); order 1: chunk i of the workgroup goes to wave i % 8.  rotate: workgroup g starts
+//                         g chunks into k and wraps round.
 // Both return 0 or a hipError_t.
 #include "skinny_gemm_args.h"
 
@@ -75,6 +79,42 @@ __global__ void __launch_bounds__(kGemmThreads) probe_weight_stream_kernel(const
         reinterpret_cast<int*>(a.D)[0] = fold[0];
 }
 
+// Packed load format: chunk c of the weight (tile-major, k fastest) is the 4 KB at c * 4096; a wave reads it with four 1 KB loads.
+__global__ void __launch_bounds__(kGemmThreads) probe_packed_stream_kernel(const GemmArgs a) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int G = a.grid;
+    const int b = blockIdx.x;
+    const int g = ((G & 7) == 0) ? (b & 7) * (G >> 3) + (b >> 3) : b;
+    const int KC = a.slabs;
+    const int t0 = g * a.rows_q + min(g, a.rows_r);          // first 16-row tile of the band
+    const int T = a.rows_q + (g < a.rows_r ? 1 : 0);
+    const int TC = T * KC;
+    const bool cyclic = a.packed == 1;
+    const int i0 = cyclic ? wv : (wv * TC) >> 3, i1 = cyclic ? TC : ((wv + 1) * TC) >> 3, step = cyclic ? kGemmWaves : 1;
+    const int rot = a.k_rotate ? g % KC : 0;
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(a.B, (uint32_t)((a.n + 15) >> 4) * (uint32_t)KC * (uint32_t)kTileBytes);
+    v4i wq[4];
+    auto issue_chunk = [&](int i) __attribute__((always_inline)) {
+        const int tile = i / KC;
+        int kc = i - tile * KC + rot;
+        if (kc >= KC) kc -= KC;
+        const uint32_t base = ((uint32_t)(t0 + tile) * (uint32_t)KC + (uint32_t)kc) * (uint32_t)kTileBytes + (uint32_t)lane * 16u;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) wq[t] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)(base + (uint32_t)t * 1024u), 0, 2 /* nt */);
+    };
+    if (i0 < i1) issue_chunk(i0);
+    v4i fold = {0, 0, 0, 0};
+    for (int i = i0; i < i1; i += step) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) fold ^= wq[t];
+        if (i + step < i1) issue_chunk(i + step);
+    }
+    if (fold[0] == 0x12345678 && fold[1] == (int)0x9abcdef0 && fold[2] == 0x0fedcba9 && fold[3] == 0x87654321)
+        reinterpret_cast<int*>(a.D)[0] = fold[0];
+}
+
 }  // namespace hfrk
 
 extern "C" {
@@ -110,6 +150,26 @@ int probe_weight_stream(const void* B, void* sink, int n, int k, int b_stride, i
     geometry(args.rows_q, &args.tiles_b, &args.base_b, &args.extra_b);
     args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)args.slabs - 1) / (uint64_t)args.slabs);
     hipLaunchKernelGGL(hfrk::probe_weight_stream_kernel, dim3(grid), dim3(hfrk::kGemmThreads), 0, static_cast<hipStream_t>(stream), args);
+    return (int)hipGetLastError();
+}
+
+int probe_packed_stream(const void* B, void* sink, int n, int k, int grid, int order, int rotate, void* stream) {
+    if (!B || !sink || n < 16 || k < 512 || k % 256 != 0 || (reinterpret_cast<uintptr_t>(B) & 15)) return (int)hipErrorInvalidValue;
+    if (((long)n + 128) * k >= (1L << 31)) return (int)hipErrorInvalidValue;
+    const int tiles = (n + 15) / 16;
+    if (grid < 1 || grid > hfrk::kMaxStreamGrid || grid > tiles) return (int)hipErrorInvalidValue;
+    hfrk::GemmArgs args = {};
+    args.B = static_cast<const uint8_t*>(B);
+    args.D = sink;
+    args.n = n;
+    args.k = k;
+    args.grid = grid;
+    args.slabs = k / 256;
+    args.rows_q = tiles / grid;
+    args.rows_r = tiles % grid;
+    args.packed = order;
+    args.k_rotate = rotate;
+    hipLaunchKernelGGL(hfrk::probe_packed_stream_kernel, dim3(grid), dim3(hfrk::kGemmThreads), 0, static_cast<hipStream_t>(stream), args);
     return (int)hipGetLastError();
 }
 

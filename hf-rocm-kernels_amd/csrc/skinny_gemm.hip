@@ -687,6 +687,49 @@ static int make_rows_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     return fill_rows_plan(m, n, k, row_tiles, (int)grid, plan);
 }
 
+// The row-split decomposition on bands of whole 16-row tiles (skinny_gemm_rows_tiled.hip), the form a weight in the packed
+// load format can take: plan wn = -3, wk = 16-row tiles per chunk, ch = activation loads, panels = 16-row tiles, slabs = k / 256.
+static int fill_rows_tiled_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk_gemm_plan* plan) {
+    const int act_loads = rows_act_loads(m);
+    if (m > kRowsMaxM || !rows_variant_exists(act_loads, row_tiles) || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
+    const long tiles = (n + 15) / 16;
+    long grid = grid_hint > 0 ? grid_hint : kNumCU;
+    if (grid > tiles) grid = tiles;
+    plan->m_tiles = 1;
+    plan->wn = -3;
+    plan->wk = row_tiles;
+    plan->ch = act_loads;
+    plan->grid = (int)grid;
+    plan->panels = (int)tiles;
+    plan->slabs = k / 256;
+    plan->lds_bytes = rows_lds_bytes(row_tiles, act_loads);
+    return HFRK_SUCCESS;
+}
+
+// Packed weights up to 16 activation rows.  Rules read off a sweep of every decomposition over the Llama-3 8B / 70B weights:
+//  * the busiest workgroup's tile count is what it is on 256 workgroups, ceil(tiles / 256); the grid is the smallest
+//    multiple of 8 from 192 on that keeps it (6144 x 4096: 384 tiles, 2 each on 192 workgroups, 6.5 us against 6.9 on 256;
+//    10240 x 8192: 640 tiles, up to 3 each on 216..240 workgroups, 15.9 us against 16.5 on 256);
+//  * two tiles per chunk from 9 rows on when a band has two, and at any row count on k above 16384 (8192 x 28672: 37.7 us
+//    against 39.4 at 8 rows);
+//  * not on the largest weights (57344 x 8192: 73.6-76.5 us against 72.8 for the workgroup kernel and 68.5 for the row-major
+//    weight -- a run of 56 contiguous chunks per wave is the slowest way to read that much memory).
+static int make_rows_tiled_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (m > 16 || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
+    const long tiles = (n + 15) / 16;
+    if (tiles < 3 * kNumCU / 4 || (long)n * k > (256L << 20)) return HFRK_INVALID_CONFIG;
+    const long busiest = (tiles + kNumCU - 1) / kNumCU;
+    long grid = (tiles + busiest - 1) / busiest;
+    grid = (grid + 7) / 8 * 8;
+    if (grid < 3 * kNumCU / 4) grid = 3 * kNumCU / 4;
+    if (grid > kNumCU) grid = kNumCU;
+    if (grid > tiles) grid = tiles;
+    if (tiles * 10 < ((tiles + grid - 1) / grid) * grid * 7) return HFRK_INVALID_CONFIG;  // busiest at most 40 % above the mean
+    const long band_tiles = (tiles + grid - 1) / grid;
+    const int row_tiles = (band_tiles >= 2 && (m >= 9 || k > 16384)) ? 2 : 1;
+    return fill_rows_tiled_plan(m, n, k, row_tiles, (int)grid, plan);
+}
+
 // 17 <= m <= 64 (valid from 1): the waves of a workgroup split K windows of 8*wave_k bytes, activations in registers
 // (skinny_gemm_ksplit.hip).  wave_k 512 keeps twice the bytes in flight and halves the window count, 256 makes
 // twice the units: take the one whose busiest workgroup streams fewer bytes.
@@ -880,7 +923,8 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
         if (chunks <= (long)kNumCU * kGemmWaves && make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         // Bands of rows per workgroup: nothing crosses workgroups and the end of the launch is short (0.3-1.3 us less than
         // the wave-stream split on every Llama-3 8B / 70B projection at 1..16 rows).
-        if (!packed && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // (row-major weights only)
+        if (!packed && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // (bands of any multiple of 4 rows: row-major weights only)
+        if (packed && make_rows_tiled_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // bands of whole 16-row tiles
         return make_stream_plan(m, n, k, plan);
     }
     // 17..32 rows in the row-split kernel (two activation tiles): every workgroup then pulls all m x k activation bytes out
@@ -929,7 +973,17 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
 }
 
 static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p, bool packed = false) {
-    if (swiglu && p->wn != 0 && p->wn != -2 && p->wn != -1) return HFRK_INVALID_CONFIG;  // the workgroup kernel has no fused epilogue
+    if (swiglu && p->wn != 0 && p->wn != -2 && p->wn != -1 && p->wn != -3) return HFRK_INVALID_CONFIG;  // the workgroup kernel has no fused epilogue
+    if (p->wn == -3) {  // row-split on bands of whole 16-row tiles, either weight layout: wk = tiles per chunk, ch = activation loads
+        if (swiglu && (p->wk != 2 || p->ch > 4)) return HFRK_INVALID_CONFIG;
+        if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
+        if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+        if (p->m_tiles != 1 || p->panels != (n + 15) / 16 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
+        if (p->grid < 1 || p->grid > kMaxStreamGrid || p->grid > p->panels) return HFRK_INVALID_CONFIG;
+        if (p->lds_bytes != rows_lds_bytes(p->wk, p->ch)) return HFRK_INVALID_CONFIG;
+        if (((long)p->panels / p->grid + 2) * p->slabs * p->slabs >= (1L << 31)) return HFRK_BAD_SHAPE;  // as below
+        return HFRK_SUCCESS;
+    }
     if (p->wn == -2) {  // row-split decomposition: wk = matrix tiles per chunk, ch = activation loads
         if (packed) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
         if (swiglu && (p->wk != 2 || p->ch > 4)) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows; up to 16 rows
@@ -1056,12 +1110,12 @@ static int choose_plan(int m, int n, int k, bool packed, hfrk_gemm_plan* plan) {
 
 // Workspace bytes and arrival counters a plan's kernel may touch (the kernels' own slot arithmetic, 1 KB per 16x16 fp32 tile).
 static size_t plan_ws_bytes(const hfrk_gemm_plan& p) {
-    if (p.wn == -2) return 0;  // row-split: nothing crosses workgroups
+    if (p.wn <= -2) return 0;  // row-split: nothing crosses workgroups
     if (p.wn == 0) return (size_t)p.grid * 2 * (p.wk * ((p.ch + 3) / 4)) * 1024;  // two slots per workgroup, row tiles x activation tiles
     if (p.wn == -1) return p.slabs > 1 ? (size_t)p.panels * p.slabs * p.m_tiles * 1024 : 0;  // one share per unit and activation tile
     return (size_t)p.grid * 2 * (p.wn * p.m_tiles) * 1024;  // two slots per workgroup, a panel's tiles x activation tiles
 }
-static long plan_counters(const hfrk_gemm_plan& p) { return p.wn == -2 ? 0 : p.wn == -1 ? (long)p.panels * p.m_tiles : p.panels; }
+static long plan_counters(const hfrk_gemm_plan& p) { return p.wn <= -2 ? 0 : p.wn == -1 ? (long)p.panels * p.m_tiles : p.panels; }
 
 // D = (base ? base : 0) + scale_a x scale_b x A.B   (epilogue 0), or the fused SwiGLU form (epilogue 1).
 // use_static: partial sums and counters go to this device's `scratch` array instead of the stream's workspace.
@@ -1145,6 +1199,8 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         } else if (swiglu && !packed && make_rows_plan(m, n / 2, k, &p) == HFRK_SUCCESS) {
             // bands of output columns; every chunk holds the gate rows and the up rows of up to 16 of them
             rc = fill_rows_plan(m, n / 2, k, 2, p.grid, &p);
+        } else if (swiglu && packed && make_rows_tiled_plan(m, n / 2, k, &p) == HFRK_SUCCESS) {
+            rc = fill_rows_tiled_plan(m, n / 2, k, 2, p.grid, &p);  // the same on bands of whole tiles of 16 output columns
         } else if (swiglu) {
             rc = fill_stream_plan(m, n / 2, k, 1, false, 0, &p);
             if (rc == HFRK_SUCCESS) {  // the chunk count of a one-tile plan over n/2 rows, but every chunk holds a gate and an up tile
@@ -1242,6 +1298,25 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
             return launch_rows_kernel(args, p.ch, p.wk, swiglu, true, rows_rms_lds_bytes(p.ch, p.wk, k), stream);
         }
         return launch_rows_kernel(args, p.ch, p.wk, swiglu, false, p.lds_bytes, stream);
+    }
+    if (p.wn == -3) {
+        const int per_tile = swiglu ? 4 : 4 * p.wk;  // units a chunk can hold
+        args.rows_q = p.panels / p.grid;            // 16-row tiles per workgroup, the first rows_r workgroups one more
+        args.rows_r = p.panels % p.grid;
+        args.tiles_a = (4 * (args.rows_q + 1) + per_tile - 1) / per_tile;
+        args.tiles_b = (4 * args.rows_q + per_tile - 1) / per_tile;
+        args.base_a = args.base_b = per_tile;
+        args.extra_a = args.extra_b = 0;
+        args.kc_magic = (uint32_t)(((1ULL << 32) + (uint64_t)p.slabs - 1) / (uint64_t)p.slabs);
+        {
+            // as for the 4-row dealing below; a packed weight is contiguous, so its bands are always a whole number of 4 KB apart
+            const int tiles = 2 * args.rows_r > p.grid ? args.tiles_a : args.tiles_b;
+            const long run8 = (long)tiles * p.slabs;
+            const bool same_offset = run8 % 8 == 0 && (run8 / 8) % 16 == 0;
+            const bool shared_lines = p.ch >= 3 && p.panels >= p.grid;
+            args.k_rotate = ((packed || b_stride % 4096 == 0) && (same_offset || shared_lines)) ? 1 : 0;
+        }
+        return launch_rows_tiled_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     }
     if (p.wn == 0) return launch_stream_kernel(args, p.ch, p.wk, swiglu, p.lds_bytes, stream);
     if (p.wn == -1) return launch_ksplit_kernel(args, p.m_tiles, p.wk * 256, swiglu, p.lds_bytes, stream);

@@ -35,7 +35,9 @@ struct GemmArgs {
     int panels, slabs, units, grid;  // units = panels * slabs
     int chunks_q, chunks_r;  // stream kernel: (panels * slabs) / grid and % grid
     // row-split kernel: 4-row units per workgroup (rows_q, the first rows_r workgroups one more), and for both band
-    // heights (a: rows_q + 1 units, b: rows_q) the tiles of a band, units per tile and how many tiles have one more
+    // heights (a: rows_q + 1 units, b: rows_q) the tiles of a band, units per tile and how many tiles have one more.
+    // On bands of whole 16-row tiles (skinny_gemm_rows_tiled.hip) rows_q / rows_r count those tiles, tiles_a / tiles_b the chunks
+    // per 256 bytes of k (up to row_tiles 16-row tiles each), and base / extra are unused.
     int rows_q, rows_r;
     int tiles_a, base_a, extra_a, tiles_b, base_b, extra_b;
     uint32_t kc_magic;       // ceil(2^32 / slabs): i / slabs == umulhi(i, kc_magic) for the chunk indices of a band
@@ -86,6 +88,9 @@ constexpr int kRowsRmsRedBytes = 8 * kGemmWaves * 4;  // per-row, per-wave parti
 constexpr int rows_rms_lds_bytes(int act_loads, int row_tiles, int k) {
     return kGemmWaves * row_tiles * kTileBytes + kRowsRmsRedBytes + 4 * act_loads * k;  // weight tiles, partial sums, [4*act_loads, k] fp8
 }
+// the same kernel on bands of whole 16-row tiles (skinny_gemm_rows_tiled.hip): args.rows_q / rows_r count 16-row tiles (with swiglu:
+// tiles of 16 output columns), args.packed selects the packed load format; no RMSNorm prologue
+int launch_rows_tiled_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream);
 constexpr int kRowsMaxM = 32;  // 17..32 rows: act_loads 6 (up to 24 rows) or 8, two matrix tiles per chunk, plain epilogue
 constexpr int rows_act_loads(int m) { return m <= 16 ? (m + 3) / 4 : m <= 24 ? 6 : 8; }
 constexpr int rows_lds_bytes(int row_tiles, int act_loads) { return kGemmWaves * (row_tiles + (act_loads + 3) / 4) * kTileBytes; }

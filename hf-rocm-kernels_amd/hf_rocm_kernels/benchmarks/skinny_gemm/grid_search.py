@@ -1,7 +1,7 @@
 """Time every decomposition the library offers for a GEMM shape and report the fastest next to the planner's choice.
 
 Counterpart of the reference package's benchmarks/skinny_gemm/grid_search.py, which walks its knob tuples
-(a_lanes, b_lanes, qsize, op_m, ops).  Here the search space is `hfrk_gemm_plan`: the wave-stream, K-split and
+(a_lanes, b_lanes, qsize, op_m, ops).  Here the search space is `hfrk_gemm_plan`: the row-split, wave-stream, K-split and
 workgroup decompositions with their parameters and a few grid sizes, passed to `hfrk_skinny_gemm_ex`.  The rules in
 the library's planner were read off sweeps like this one; `--save table.json` writes the winners that beat the planner
 as a plan table (hf_rocm_kernels/plan_table.py: load it, or point HFRK_PLAN_TABLE at it).  The sweep itself runs with
@@ -54,6 +54,10 @@ def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.Gemm
         for rt in ((1, 2) if m <= 16 else (2,)):
             for g in wide:
                 plans.append(_capi.GemmPlan(1, -2, rt, ma, min(g, units), units, k // 256, 8 * (rt + (ma + 3) // 4) * 4096))
+        tiles = -(-n // 16)  # the same on bands of whole 16-row tiles: the form that also reads the packed load format
+        for rt in ((1, 2) if m <= 16 else (2,)):
+            for g in wide:
+                plans.append(_capi.GemmPlan(1, -3, rt, ma, min(g, tiles), tiles, k // 256, 8 * (rt + (ma + 3) // 4) * 4096))
     for wave_k in (256, 512, 1024):  # K-split
         if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
             tiles, windows = -(-n // 16), k // (8 * wave_k)
@@ -77,6 +81,8 @@ def candidate_plans(m: int, n: int, k: int, grids: List[int]) -> List[_capi.Gemm
 def describe(p: _capi.GemmPlan) -> str:
     if p.wn == -2:
         return f"row-split row_tiles={p.wk} act_loads={p.ch} grid={p.grid}"
+    if p.wn == -3:
+        return f"row-split-tiles row_tiles={p.wk} act_loads={p.ch} grid={p.grid}"
     if p.wn == 0:
         return f"wave-stream row_tiles={p.wk} act_loads={p.ch} grid={p.grid}"
     if p.wn == -1:
@@ -143,6 +149,7 @@ def main() -> None:
                         help="write a plan table (hf_rocm_kernels.plan_table) of the winners that beat the planner by --min-gain")
     parser.add_argument("--min-gain", type=float, default=0.03, help="relative gain a winner needs to enter the plan table")
     args = parser.parse_args()
+    from hf_rocm_kernels import plan_table
     lib = _capi.load()
     _capi.check(lib.hfrk_init(), "hfrk_init")
     arena = torch.randint(0, 120, (1 << 30,), dtype=torch.uint8, device="cuda")  # finite fp8 codes
@@ -152,7 +159,7 @@ def main() -> None:
         if n < MIN_ROWS:
             print(f"m={m} n={n} k={k}: skipped (this tool does not run weights under {MIN_ROWS} rows, see the note at the top)")
             continue
-        chosen = _capi.plan(m, n, k)
+        chosen = plan_table.get_plan(m, n, k, packed=args.packed)  # (with HFRK_PLAN_TABLE=none: the planner's own choice)
         t_default = time_plan(lib, arena, m, n, k, None, args.reps, args.packed)
         rows = []
         for p in candidate_plans(m, n, k, args.grids):
@@ -176,7 +183,6 @@ def main() -> None:
         table[f"{m}x{n}x{k}"] = {"planner": chosen.as_dict(), "planner_us": t_default,
                                  "plans": [{"us": t, "plan": d} for t, _, d in rows]}
     if args.save:
-        from hf_rocm_kernels import plan_table
         plan_table.save(winners, args.save)
         print(f"wrote {len(winners)} entries to {args.save}")
     if args.json:

@@ -64,7 +64,10 @@ enum hfrk_weight_format { HFRK_WEIGHT_E4M3FN = 0, HFRK_WEIGHT_E4M3FNUZ = 1 };
 typedef struct hfrk_gemm_plan {
     int m_tiles;   /* ceil(m/16): 16-row activation tiles (wave-stream: 1..2, others: 1..4; row-split: always 1, the kernel takes its tiles from ch) */
     int wn;        /* which decomposition:
-                      -2          row-split (m <= 32, k >= 512): every workgroup owns a band of weight rows and all of k
+                      -2          row-split (m <= 32, k >= 512): every workgroup owns a band of weight rows and all of k;
+                                  bands of any number of 4-row units, row-major weights only
+                      -3          the same on bands of whole 16-row tiles: row-major weights and the packed load format
+                                  (same bits from both)
                        0          wave-stream (m <= 32): every wave streams its own run of chunks
                       -1          K-split (k % (2048*wk) == 0): the 8 waves of a workgroup split K, activations in registers
                        1..16      workgroup: a panel is wn 16-row weight tiles; the 8 waves are 8/wk row waves x wk K waves,
@@ -77,7 +80,7 @@ typedef struct hfrk_gemm_plan {
                       6 up to 24 rows, else 8).  K-split: 0 */
     int grid;      /* persistent workgroups launched */
     int panels;    /* workgroup: ceil(n / (16*wn)) row panels.  wave-stream: ceil(n / (16*wk)) row groups.
-                      K-split: ceil(n/16) row tiles.  row-split: ceil(n/4) units of 4 rows */
+                      K-split: ceil(n/16) row tiles.  row-split: ceil(n/4) units of 4 rows (wn = -3: ceil(n/16) tiles) */
     int slabs;     /* workgroup: k / (256*wk*ch) K slabs per panel.  wave-stream: k/256 chunks per group.
                       K-split: k / (2048*wk) windows */
     int lds_bytes; /* dynamic LDS per workgroup */

@@ -289,7 +289,8 @@ def audit_rows(m, n, k, b_stride, p, swiglu=False):
     assert 8 * wave_lds == p.lds_bytes <= 160 * 1024
     assert MT * RT * 64 * 16 <= RT * TILE   # a wave's partial sums fit the start of its own weight tiles
     # (SwiGLU: n counts the output columns; the weight has 2n rows, gate rows first)
-    w = Buf("weights", ((2 * n if swiglu else n) - 1) * b_stride + k)
+    n_rows = 2 * n if swiglu else n
+    w = Buf("weights", (n_rows - 1) * b_stride + k)
     a = Buf("activations", m * k)
     q, r = divmod(units, G)
     xcd_ids(G)
@@ -321,9 +322,62 @@ def audit_rows(m, n, k, b_stride, p, swiglu=False):
     return w.hits
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# row-split kernel on bands of whole 16-row tiles (skinny_gemm_rows_tiled.hip), row-major and packed weights
+def audit_tiles(m, n, k, b_stride, p, swiglu=False, packed=False):
+    RT, MA = p.wk, p.ch
+    MT = (MA + 3) // 4
+    G, tiles, KC = p.grid, p.panels, p.slabs
+    PT = 4 if swiglu else 4 * RT       # 4-row units per chunk
+    assert tiles == (n + 15) // 16 and KC == k // 256 and k % 256 == 0 and k >= 512 and G <= min(tiles, 512) and 4 * MA >= m
+    wave_lds = (RT + MT) * TILE
+    assert 8 * wave_lds == p.lds_bytes <= 160 * 1024
+    assert MT * RT * 64 * 16 <= RT * TILE   # a wave's partial sums fit the start of its own weight tiles
+    n_rows = 2 * n if swiglu else n
+    w = Buf("weights", ((n_rows + 15) >> 4) * KC * TILE if packed else (n_rows - 1) * b_stride + k)
+    a = Buf("activations", m * k)
+    q, r = divmod(tiles, G)
+    xcd_ids(G)
+    for g in range(G):
+        nt, t0 = q + (1 if g < r else 0), g * q + min(g, r)
+        band_units, u0 = 4 * nt, 4 * t0
+        T = -(-band_units // PT)
+        TC = T * KC
+        for wv in range(8):
+            i0, i1 = (wv * TC) >> 3, ((wv + 1) * TC) >> 3
+            for i in {i0, i1 - 1} if i1 > i0 else ():
+                j, kc = divmod(i, KC)
+                units, row0 = min(PT, band_units - PT * j), 4 * (u0 + PT * j)
+                assert units >= 4 and units % 4 == 0 and row0 % 16 == 0
+                for rot in (0, g % KC):
+                    kr = (kc + rot) % KC
+                    for li, lg in LANES:
+                        for t in (0, MA - 1):
+                            a.access(lg * k + li * 16 + kr * 256 + 4 * t * k, 16, 4 * t + lg < m)
+                        for t in range(4 * RT):
+                            if packed:   # piece t % 4 of 16-row tile t // 4 of the chunk
+                                tile16 = (row0 >> 4) + (t // 4) * ((2 * n) >> 5 if swiglu else 1)
+                                if swiglu or 4 * (t // 4) < units:
+                                    w.access((tile16 * KC + kr) * TILE + (t % 4) * 1024 + (lg * 16 + li) * 16, 16, True)
+                                else:
+                                    w.access(OOR, 16, False)
+                            else:
+                                unit = t % 4 if swiglu else t
+                                rowoff = 4 * unit + (t // 4) * n if swiglu else 4 * t
+                                row = row0 + rowoff + lg
+                                if unit < units:
+                                    w.access(lg * b_stride + li * 16 + (row0 + rowoff) * b_stride + kr * 256, 16,
+                                             row - (t // 4) * n < n if swiglu else row < n)
+                                else:
+                                    w.access(lg * b_stride + li * 16 + OOR, 16, False)
+    return w.hits
+
+
 def audit(m, n, k, p, packed=False):
     if p.wn == -2:
         return audit_rows(m, n, k, k, p)
+    if p.wn == -3:
+        return audit_tiles(m, n, k, k, p, packed=packed)
     if p.wn == 0:
         return audit_stream(m, n, k, k, p, packed)
     if p.wn == -1:
@@ -395,6 +449,11 @@ def test_planner_and_forced_plans_stay_inside_their_buffers(m, n, k):
         assert audit(m, n, k, p) > 0, p.as_dict()
         if p.wn != -2 and k % 256 == 0:
             assert audit(m, n, k, p, packed=True) > 0, p.as_dict()
+    if k % 256 == 0 and m <= 16:
+        lib = _capi.load()
+        p = _capi.GemmPlan()
+        assert lib.hfrk_plan_table_get(m, n, k, 1, ctypes.byref(p)) == _capi.SUCCESS   # the planner's answer for a packed weight
+        assert audit(m, n, k, p, packed=True) > 0, p.as_dict()
 
 
 def test_k_that_ends_inside_a_chunk_and_padded_row_strides():
@@ -404,7 +463,7 @@ def test_k_that_ends_inside_a_chunk_and_padded_row_strides():
     assert audit(3, 130, 144, p) > 0
     for m, n, k, stride in [(8, 1000, 1024, 1024 + 256), (32, 512, 2048, 4096), (64, 777, 4096, 4096 + 16)]:
         p = _capi.plan(m, n, k)
-        fn = {-2: audit_rows, 0: audit_stream, -1: audit_ksplit}.get(p.wn, audit_workgroup)
+        fn = {-2: audit_rows, -3: audit_tiles, 0: audit_stream, -1: audit_ksplit}.get(p.wn, audit_workgroup)
         assert fn(m, n, k, stride, p) > 0
 
 
@@ -414,6 +473,10 @@ def test_swiglu_bands_of_the_row_split_kernel():
         units = -(-n_out // 4)
         p = _capi.GemmPlan(1, -2, 2, (m + 3) // 4, min(256, units), units, k // 256, 8 * 3 * 4096)
         assert audit_rows(m, n_out, k, k, p, swiglu=True) > 0
+        tiles = -(-n_out // 16)
+        p = _capi.GemmPlan(1, -3, 2, (m + 3) // 4, min(200, tiles), tiles, k // 256, 8 * 3 * 4096)
+        assert audit_tiles(m, n_out, k, k, p, swiglu=True) > 0
+        assert audit_tiles(m, n_out, k, k, p, swiglu=True, packed=True) > 0
 
 
 def test_library_refuses_grids_no_test_covers():
@@ -441,4 +504,4 @@ def test_library_refuses_grids_no_test_covers():
     import inspect
     assert "small-weights" not in inspect.getsource(grid_search)
     for p in grid_search.candidate_plans(m, 4096, k, [192, 512, 1024]):
-        assert p.grid <= (512 if p.wn in (0, -2) else 256)
+        assert p.grid <= (512 if p.wn in (0, -2, -3) else 256)

@@ -71,6 +71,10 @@ def all_plans(m, n, k):
         for rt in ((1, 2) if m <= 16 else (2,)):
             for grid in sorted({min(g, units) for g in (256, 200, 7, 512, 1, 77)}):
                 plans.append(_capi.GemmPlan(1, -2, rt, ma, grid, units, k // 256, 8 * (rt + (ma + 3) // 4) * 4096))
+        tiles = (n + 15) // 16  # the same on bands of whole 16-row tiles (the form that also reads the packed load format)
+        for rt in ((1, 2) if m <= 16 else (2,)):
+            for grid in sorted({min(g, tiles) for g in (256, 200, 7, 384, 1, 77)}):
+                plans.append(_capi.GemmPlan(1, -3, rt, ma, grid, tiles, k // 256, 8 * (rt + (ma + 3) // 4) * 4096))
     for wave_k in (256, 512, 1024):  # K-split decomposition
         if k % (8 * wave_k) == 0 and (wave_k < 1024 or mt <= 2):
             tiles, windows = (n + 15) // 16, k // (8 * wave_k)
@@ -592,6 +596,30 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
         f = out.cpu().float()
         assert not f.isnan().any(), ("rows", grid)
         assert ((f - ref.float()).abs() <= tol).all(), ("rows", grid)
+    # the same on bands of whole tiles of 16 output columns, from the row-major and from the packed weight
+    from hf_rocm_kernels.utils.weight_format import pack_weight
+    packed = pack_weight(w.t())
+    tiles = (n // 2 + 15) // 16
+    for grid in sorted({min(g, tiles) for g in (384, 256, 200, 64, 7, 1)}):
+        plan = _capi.GemmPlan(1, -3, 2, ma, grid, tiles, kc, 8 * 3 * 4096)
+        outs = []
+        for layout in ("row-major", "packed"):
+            out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
+            if layout == "packed":
+                st = lib.hfrk_skinny_gemm_packed(a.data_ptr(), packed.data.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                                                 out_scale.data_ptr(), m, n, k, _capi.BF16, _capi.EPILOGUE_SWIGLU, ctypes.byref(plan),
+                                                 torch.cuda.current_stream().cuda_stream)
+            else:
+                st = lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
+                                                out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
+                                                ctypes.byref(plan), torch.cuda.current_stream().cuda_stream)
+            assert st == 0, ("rows on tiles", layout, grid, st)
+            torch.cuda.synchronize()
+            f = out.cpu().float()
+            assert not f.isnan().any(), ("rows on tiles", layout, grid)
+            assert ((f - ref.float()).abs() <= tol).all(), ("rows on tiles", layout, grid)
+            outs.append(out.view(torch.uint8))
+        assert torch.equal(outs[0], outs[1]), ("rows on tiles: the two layouts differ", grid)
     one_tile = _capi.GemmPlan(1, -2, 1, ma, 64, units, kc, 8 * 2 * 4096)  # a chunk must hold a gate and an up tile
     assert lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
                                       out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,

@@ -122,13 +122,18 @@ def _emulate_rows(plan):
     whose partials it adds).  Returns nothing; asserts that every (unit, K chunk) is multiplied exactly once and every
     tile is finished exactly once from exactly the partials that exist."""
     G, units, KC, per_tile = plan.grid, plan.panels, plan.slabs, 4 * plan.wk
-    q, r = divmod(units, G)
+    tiled = plan.wn == -3   # bands of whole 16-row tiles (plan.panels counts them): chunks of per_tile units, a last one of fewer
+    if tiled:
+        units *= 4
+    q, r = divmod(plan.panels, G)
     magic = ((1 << 32) + KC - 1) // KC
     assert magic < (1 << 32)
     cover = [[0] * KC for _ in range(units)]
     for g in range(G):
         nu, u0 = q + (1 if g < r else 0), g * q + min(g, r)
         assert nu >= 1, "empty workgroup"
+        if tiled:
+            nu, u0 = 4 * nu, 4 * u0
         T = -(-nu // per_tile)
         base, extra = nu // T, nu % T
         TC = T * KC
@@ -141,12 +146,14 @@ def _emulate_rows(plan):
             for i in range(i0, i1):
                 j, kc = divmod(i, KC)
                 first, height = j * base + min(j, extra), base + (1 if j < extra else 0)
+                if tiled:
+                    first, height = per_tile * j, min(per_tile, nu - per_tile * j)
                 assert 1 <= height <= per_tile
                 for t in range(height):
                     cover[u0 + first + t][kc] += 1
                 if not pieces[j] or pieces[j][-1] != w:
                     pieces[j].append(w)
-        assert sum(base + (1 if j < extra else 0) for j in range(T)) == nu
+        assert tiled or sum(base + (1 if j < extra else 0) for j in range(T)) == nu
         finished = [0] * T
         for w, (i0, i1) in enumerate(runs):
             count, kb0 = i1 - i0, i0 % KC
@@ -178,6 +185,14 @@ def test_row_split_decomposition_on_the_host(n, k, grid, rt):
     plan = _capi.GemmPlan(1, -2, rt, 2, min(grid, units), units, k // 256, 8 * (rt + 1) * 4096)
     assert _capi.load().hfrk_plan_table_set(8, n, k, 0, ctypes.byref(plan)) == _capi.SUCCESS   # the library accepts it
     assert _capi.load().hfrk_plan_table_set(8, n, k, 0, None) == _capi.SUCCESS
+    assert _capi.load().hfrk_plan_table_set(8, n, k, 1, ctypes.byref(plan)) == _capi.INVALID_CONFIG   # not for the packed load format
+    _emulate_rows(plan)
+    # the same on bands of whole 16-row tiles, the form both weight layouts take
+    tiles = -(-n // 16)
+    plan = _capi.GemmPlan(1, -3, rt, 2, min(grid, tiles), tiles, k // 256, 8 * (rt + 1) * 4096)
+    for packed in (0, 1):
+        assert _capi.load().hfrk_plan_table_set(8, n, k, packed, ctypes.byref(plan)) == _capi.SUCCESS
+        assert _capi.load().hfrk_plan_table_set(8, n, k, packed, None) == _capi.SUCCESS
     _emulate_rows(plan)
 
 
@@ -256,10 +271,11 @@ def test_planner_on_random_shapes_gives_plans_the_launcher_accepts_and_that_cove
             assert lib.hfrk_plan_table_set(m, n, k, int(packed), ctypes.byref(p)) == _capi.SUCCESS, (m, n, k, packed, p.as_dict())
             plan_table.clear()
             assert not packed or p.wn != -2  # bands of any 4-row height do not exist in 16-row packed tiles
+            assert packed or p.wn != -3      # (the planner deals row-major weights in 4-row units)
             kinds.add(p.wn if p.wn <= 0 else 1)
             if p.panels * p.slabs > 200000:
                 continue  # (the replay is a Python loop over units)
-            if p.wn == -2:
+            if p.wn in (-2, -3):
                 _emulate_rows(p)
             elif p.wn == 0:
                 assert all(c == 1 for c in _emulate_stream(p)[0]), (m, n, k)
@@ -270,7 +286,7 @@ def test_planner_on_random_shapes_gives_plans_the_launcher_accepts_and_that_cove
                 assert all(c == 1 for row in _emulate(p, n, k)[0] for c in row), (m, n, k)
     finally:
         plan_table.clear()
-    assert kinds == {-2, -1, 0, 1}
+    assert kinds == {-3, -2, -1, 0, 1}
 
 
 def test_plan_rejects_what_the_kernel_cannot_take():
@@ -605,7 +621,7 @@ def test_every_plan_the_sweep_tool_proposes_is_one_the_library_accepts(m, n, k):
             status = _capi.load().hfrk_plan_table_set(m, n, k, 0, ctypes.byref(p))
             assert status == _capi.SUCCESS, (grid_search.describe(p), p.as_dict(), _capi.status_string(status))
             families.add(grid_search.describe(p).split()[0])
-            if p.wn == -2:
+            if p.wn in (-2, -3):
                 _emulate_rows(p)
             elif p.wn == 0:
                 assert all(c == 1 for c in _emulate_stream(p)[0]), grid_search.describe(p)
