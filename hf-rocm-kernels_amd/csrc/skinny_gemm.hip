@@ -975,7 +975,7 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
 static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p, bool packed = false) {
     if (swiglu && p->wn != 0 && p->wn != -2 && p->wn != -1 && p->wn != -3) return HFRK_INVALID_CONFIG;  // the workgroup kernel has no fused epilogue
     if (p->wn == -3) {  // row-split on bands of whole 16-row tiles, either weight layout: wk = tiles per chunk, ch = activation loads
-        if (swiglu && (p->wk != 2 || p->ch > 4)) return HFRK_INVALID_CONFIG;
+        if (swiglu && p->wk != 2) return HFRK_INVALID_CONFIG;
         if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
         if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
         if (p->m_tiles != 1 || p->panels != (n + 15) / 16 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
@@ -986,7 +986,7 @@ static int check_plan(int m, int n, int k, bool swiglu, const hfrk_gemm_plan* p,
     }
     if (p->wn == -2) {  // row-split decomposition: wk = matrix tiles per chunk, ch = activation loads
         if (packed) return HFRK_INVALID_CONFIG;  // bands of any 4-row height do not fit the packed format's 16-row tiles
-        if (swiglu && (p->wk != 2 || p->ch > 4)) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows; up to 16 rows
+        if (swiglu && p->wk != 2) return HFRK_INVALID_CONFIG;  // n counts output columns; a chunk holds their gate and their up rows
         if (m > kRowsMaxM || !rows_variant_exists(p->ch, p->wk) || 4 * p->ch < m || k < 512) return HFRK_INVALID_CONFIG;
         if (k % 256 != 0) return HFRK_K_NOT_DIVISIBLE_BY_WARPTILE_K;
         if (p->m_tiles != 1 || p->panels != (n + 3) / 4 || p->slabs != k / 256) return HFRK_INVALID_CONFIG;
@@ -1153,8 +1153,9 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
     if ((sa_stride != 0 && sa_stride != 1) || (sb_stride != 0 && sb_stride != 1)) return HFRK_BAD_SHAPE;
     if (epilogue != HFRK_EPILOGUE_NONE && epilogue != HFRK_EPILOGUE_SWIGLU) return HFRK_INVALID_CONFIG;
     const bool swiglu = epilogue == HFRK_EPILOGUE_SWIGLU;
-    // SwiGLU epilogue: up to 16 rows in the wave-stream / row-split kernels; above, in the K-split kernel when one window covers K
-    if (swiglu && (!out_scale || base || n % 32 != 0 || (m > 16 && k != 2048 && k != 4096))) return HFRK_BAD_SHAPE;
+    // SwiGLU epilogue: up to 16 rows in the wave-stream / row-split kernels; above, in the K-split kernel when one window covers K,
+    // and up to 32 rows in the row-split kernel (two activation tiles) on any k it takes
+    if (swiglu && (!out_scale || base || n % 32 != 0 || (m > kRowsMaxM && k != 2048 && k != 4096))) return HFRK_BAD_SHAPE;
     // every offset the kernel forms, including rows of the last (padded) panel, must stay below 2^31
     if (((long)n + 128) * b_stride + k >= (1L << 31) || (long)m * k >= (1L << 31)) return HFRK_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15 || (b_stride & 15)) return HFRK_BAD_ALIGNMENT;
@@ -1194,8 +1195,12 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         if (rc != HFRK_SUCCESS) return rc;
     } else {
         int rc;
-        if (swiglu && m > 16) {
+        if (swiglu && m > 16 && (k == 2048 || k == 4096)) {
             rc = make_ksplit_plan(m, n / 2, k, &p);  // tiles of 16 output columns; a gate and an up pass per tile
+        } else if (swiglu && m > 16) {
+            // 17..32 rows on other k: bands of output columns in the row-split kernel, two activation tiles (row-major weights whose
+            // columns deal out over the workgroups; callers run the two kernels where this returns HFRK_BAD_SHAPE)
+            rc = (!packed && m <= kRowsMaxM && make_rows_plan(m, n / 2, k, &p) == HFRK_SUCCESS) ? fill_rows_plan(m, n / 2, k, 2, p.grid, &p) : HFRK_BAD_SHAPE;
         } else if (swiglu && !packed && make_rows_plan(m, n / 2, k, &p) == HFRK_SUCCESS) {
             // bands of output columns; every chunk holds the gate rows and the up rows of up to 16 of them
             rc = fill_rows_plan(m, n / 2, k, 2, p.grid, &p);

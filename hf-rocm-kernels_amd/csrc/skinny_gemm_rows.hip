@@ -14,8 +14,9 @@ int launch_rows_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool 
         return swiglu ? launch_rows_one<2, 2, true, true>(args, lds_bytes, stream) : launch_rows_one<2, 1, false, true>(args, lds_bytes, stream);
     }
     if (lds_bytes != rows_lds_bytes(row_tiles, act_loads)) return HFRK_INVALID_CONFIG;
-    if (act_loads > 4) {  // 17..32 rows: two activation tiles, two weight tiles per chunk, plain epilogue
-        if (swiglu || row_tiles != 2) return HFRK_INVALID_CONFIG;
+    if (act_loads > 4) {  // 17..32 rows: two activation tiles, two weight tiles per chunk
+        if (row_tiles != 2) return HFRK_INVALID_CONFIG;
+        if (swiglu) return act_loads == 6 ? launch_rows_one<6, 2, true, false>(args, lds_bytes, stream) : launch_rows_one<8, 2, true, false>(args, lds_bytes, stream);
         return act_loads == 6 ? launch_rows_one<6, 2, false, false>(args, lds_bytes, stream) : launch_rows_one<8, 2, false, false>(args, lds_bytes, stream);
     }
 #define HFRK_ROWS_CASE(MA_)                                                                     \

@@ -80,24 +80,28 @@ struct RowsEpilogue {
     // scale, add D (accumulate mode), round once, store: acc[mt * RT + rt]
     __device__ __forceinline__ void store(int row0, int units, const v4f (&acc)[MT * RT], const Pre& pre) const {
         if constexpr (SWIGLU) {
-            // acc[0] = gate, acc[1] = up of output columns n0 .. n0+3.  The unfused chain stores both projections in the
-            // 16-bit dtype between its two kernels: round them the same way before the activation.
-            const float sa = sa_mt[0];
+            // acc[mt * RT] = gate, acc[mt * RT + 1] = up of output columns n0 .. n0+3 of activation tile mt.  The unfused chain stores
+            // both projections in the 16-bit dtype between its two kernels: round them the same way before the activation.
             const int n0 = row0 + 4 * lg;
             const v4f sbg = __builtin_bit_cast(v4f, pre.sb[0]), sbu = __builtin_bit_cast(v4f, pre.sb[RT - 1]);
-            float y[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                float g = acc[0][v] * (sa * (per_channel ? sbg[v] : 1.0f));
-                float u = acc[RT - 1][v] * (sa * (per_channel ? sbu[v] : 1.0f));
-                g = bf16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(g)) : load16<HFRK_F16>(store16<HFRK_F16>(g));
-                u = bf16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(u)) : load16<HFRK_F16>(store16<HFRK_F16>(u));
-                y[v] = silu_mul(g, u, inv_out_scale);
+            for (int mt = 0; mt < MT; ++mt) {
+                const float sa = sa_mt[mt];
+                const int arow = 16 * mt + li;
+                float y[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    float g = acc[mt * RT][v] * (sa * (per_channel ? sbg[v] : 1.0f));
+                    float u = acc[mt * RT + RT - 1][v] * (sa * (per_channel ? sbu[v] : 1.0f));
+                    g = bf16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(g)) : load16<HFRK_F16>(store16<HFRK_F16>(g));
+                    u = bf16 ? load16<HFRK_BF16>(store16<HFRK_BF16>(u)) : load16<HFRK_F16>(store16<HFRK_F16>(u));
+                    y[v] = silu_mul(g, u, inv_out_scale);
+                }
+                uint32_t packed = cvt_pk_fp8(y[0], y[1], 0u, false);
+                packed = cvt_pk_fp8(y[2], y[3], packed, true);
+                const bool live = arow < a.m && lg < units && n0 < n_out;
+                __builtin_amdgcn_raw_buffer_store_b32((int)packed, d_rsrc, live ? (int)((uint32_t)arow * (uint32_t)n_out + (uint32_t)n0) : (int)kOutOfRange, 0, 0);
             }
-            uint32_t packed = cvt_pk_fp8(y[0], y[1], 0u, false);
-            packed = cvt_pk_fp8(y[2], y[3], packed, true);
-            const bool live = li < a.m && lg < units && n0 < n_out;
-            __builtin_amdgcn_raw_buffer_store_b32((int)packed, d_rsrc, live ? (int)((uint32_t)li * (uint32_t)n_out + (uint32_t)n0) : (int)kOutOfRange, 0, 0);
             return;
         }
 #pragma unroll

@@ -39,8 +39,8 @@
 namespace hfrk {
 
 // MA = ceil(m/4): 16-byte activation loads per lane and chunk (rows 4t .. 4t+3), RT = 16-row matrix tiles per chunk.
-// MA = 6 or 8 (17..32 rows, RT = 2, plain epilogue): the activation rows fill two 16-row tiles, and every weight operand
-// read from LDS feeds one matrix instruction per activation tile.
+// MA = 6 or 8 (17..32 rows, RT = 2): the activation rows fill two 16-row tiles, and every weight operand read from LDS
+// feeds one matrix instruction per activation tile.
 // SWIGLU: the weight is a gate_up projection (gate rows [0, n/2), up rows [n/2, n)).  Bands, units and tiles then count
 // output columns (n/2 of them); a chunk pairs up to 16 gate rows with the up rows of the same columns (RT = 2: the gate
 // tile and the up tile), and the epilogue stores e4m3fn(silu(gate) * up / out_scale) into D [m, n/2] instead of the two
@@ -70,7 +70,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     static_assert(!SWIGLU || RT == 2, "the SwiGLU epilogue pairs one gate tile with one up tile");
     static_assert(!RMS || MA <= 2, "the RMSNorm prologue keeps every row in registers: up to 8 rows");
     constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles: 2 from 17 rows on (plain epilogue, two matrix tiles per chunk)
-    static_assert(MT == 1 || (MT == 2 && RT == 2 && !SWIGLU && !RMS), "above 16 rows: two weight tiles per chunk, plain epilogue");
+    static_assert(MT == 1 || (MT == 2 && RT == 2 && !RMS), "above 16 rows: two weight tiles per chunk, no RMSNorm prologue");
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kWaveLds = (RMS ? RT : RT + MT) * kTileBytes;  // RT weight tiles, MT activation tiles (RMS: rows staged once instead)
     constexpr int R = 4 * MA;                                  // activation rows the MA loads (or the staged block) hold

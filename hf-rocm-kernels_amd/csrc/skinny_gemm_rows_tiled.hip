@@ -8,8 +8,10 @@ namespace hfrk {
 
 template <int LAYOUT>
 static int launch_rows_tiled_layout(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream) {
-    if (act_loads > 4) {  // 17..32 rows: two activation tiles, two weight tiles per chunk, plain epilogue
-        if (swiglu || row_tiles != 2) return HFRK_INVALID_CONFIG;
+    if (act_loads > 4) {  // 17..32 rows: two activation tiles, two weight tiles per chunk
+        if (row_tiles != 2) return HFRK_INVALID_CONFIG;
+        if (swiglu) return act_loads == 6 ? launch_rows_one<6, 2, true, false, LAYOUT>(args, lds_bytes, stream)
+                                          : launch_rows_one<8, 2, true, false, LAYOUT>(args, lds_bytes, stream);
         return act_loads == 6 ? launch_rows_one<6, 2, false, false, LAYOUT>(args, lds_bytes, stream)
                               : launch_rows_one<8, 2, false, false, LAYOUT>(args, lds_bytes, stream);
     }

@@ -220,13 +220,14 @@ def skinny_gemm_swiglu(
     """gate_up projection and SwiGLU in one launch: with [gate | up] = scale_a * scale_b * (skinny_a @ gate_up_weight)
     rounded to `intermediate_dtype`, returns float8_e4m3fn(silu(gate) * up / out_scale) of shape (m, n/2) -- what
     `skinny_gemm` followed by `swiglu` produces, without the (m, n) intermediate and the second launch.
-    One launch for n % 32 == 0 and m <= 16, or m <= 64 on k = 2048 / 4096 (`hfrk_skinny_gemm_fused`'s conditions); other
-    shapes run the two kernels."""
+    One launch for n % 32 == 0 and m <= 16, m <= 64 on k = 2048 / 4096, or m <= 32 on row-major weights of at least 1024 output
+    columns (`hfrk_skinny_gemm_fused`'s conditions); other shapes run the two kernels."""
     m, n = skinny_a.size(0), gate_up_weight.size(1)
     assert n % 2 == 0, f"Expected an even number of gate_up columns but got {n}"
     assert intermediate_dtype in _OUT_DTYPES, f"Expected one of {_OUT_DTYPES} but got {intermediate_dtype = }"
     assert out_scale.numel() == 1 and out_scale.dtype == torch.float32, "Expected out_scale to be one float32"
-    if n % 32 != 0 or (m > 16 and skinny_a.size(1) not in (2048, 4096)):
+
+    def two_launches() -> Tensor:
         from ..swiglu import swiglu
         gate_up = skinny_gemm_scaled(skinny_a, gate_up_weight, scale_a,
                                      scale_b if scale_b is not None else torch.ones(1, device=skinny_a.device),
@@ -236,6 +237,18 @@ def skinny_gemm_swiglu(
             return result
         output.copy_(result)
         return output
+
+    k = skinny_a.size(1)
+    if n % 32 != 0 or (m > 32 and k not in (2048, 4096)):
+        return two_launches()
+    # 17..32 rows on other k: one launch where the library's row-split kernel takes the shape (row-major weights whose
+    # output columns deal out over the workgroups), which its status says -- and where it is the faster way: measured on
+    # k = 8192 at 20 / 32 rows, 16384 columns 25.8 / 26.5 us fused against 26.0 / 26.1 in two launches, 28672 columns 44.0 /
+    # 46.4 against 40.7 / 41.0, 57344 columns 78.3 / 84.4 against 77.3 / 78.0 (above 16 rows the workgroup kernel is the
+    # faster GEMM on large weights, by more than the SwiGLU launch costs)
+    maybe = m > 16 and k not in (2048, 4096)
+    if maybe and (isinstance(gate_up_weight, PackedWeight) or torch.compiler.is_compiling() or n * k > (128 << 20)):
+        return two_launches()
     if output is None:
         output = torch.empty(size=(m, n // 2), dtype=torch.float8_e4m3fn, device=skinny_a.device)
     assert output.shape == (m, n // 2) and output.dtype == torch.float8_e4m3fn and output.is_contiguous(), (
@@ -243,8 +256,14 @@ def skinny_gemm_swiglu(
     skinny_gemm_checks(skinny_a, gate_up_weight, scale_a.reshape(-1)[:1],
                        _ShapeOnly(m, n, intermediate_dtype, skinny_a.device))
     sa, sb = _scale_vectors(skinny_a, gate_up_weight, scale_a, scale_b)
-    _fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU,
-           _capi.BF16 if intermediate_dtype == torch.bfloat16 else _capi.F16)
+    dtype_tag = _capi.BF16 if intermediate_dtype == torch.bfloat16 else _capi.F16
+    if maybe:
+        status = _skinny_gemm_fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU, dtype_tag)
+        if status == _capi.BAD_SHAPE:
+            return two_launches()
+        _raise_on_status(status, "skinny_gemm_fused")
+        return output
+    _fused(skinny_a, gate_up_weight, output, None, sa, sb, out_scale, _capi.EPILOGUE_SWIGLU, dtype_tag)
     return output
 
 

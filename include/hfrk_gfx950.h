@@ -199,8 +199,10 @@ int hfrk_skinny_gemm_noalloc(const void* A, const void* B, void* D, const float*
  *   epilogue HFRK_EPILOGUE_SWIGLU: B is a gate_up weight, gate rows [0, n/2), up rows [n/2, n);
  *       D[i,j] = e4m3fn( silu(g) * u / out_scale[0] ),  g, u = the two projections of column j, each rounded to
  *       d_dtype first (what the unfused chain stores between its two kernels);  D is fp8 [m, n/2], 4-byte aligned.
- *       Needs n % 32 == 0, base == NULL and m <= 16, or m <= 64 with k = 2048 or 4096 (the K-split kernel, whose one
- *       window then covers k); otherwise HFRK_BAD_SHAPE (callers then run the two kernels).
+ *       Needs n % 32 == 0, base == NULL and m <= 16; or m <= 64 with k = 2048 or 4096 (the K-split kernel, whose one
+ *       window then covers k); or m <= 32 on a row-major weight whose n/2 output columns deal out over the workgroups
+ *       (the row-split kernel with two activation tiles: k % 256 == 0, at least 1024 columns).  Otherwise HFRK_BAD_SHAPE
+ *       (callers then run the two kernels).
  * Scales and plan as in hfrk_skinny_gemm_ex; a plan passed with the SwiGLU epilogue describes n/2 output columns
  * with wk = 2. */
 int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,

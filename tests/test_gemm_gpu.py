@@ -466,7 +466,8 @@ def _swiglu_oracle(a, w, sa, sb, out_scale, dtype):
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("m,n,k", [(1, 512, 1024), (5, 2080, 512), (8, 28672, 4096), (13, 1024, 2048), (16, 28672, 4096),
                                    (16, 64, 256), (17, 1024, 4096), (32, 28672, 4096), (40, 4160, 2048), (64, 2048, 2048),
-                                   (64, 28672, 4096), (8, 1024, 640), (3, 4160, 4096 + 128)])
+                                   (64, 28672, 4096), (8, 1024, 640), (3, 4160, 4096 + 128),
+                                   (32, 16384, 8192), (20, 4160, 3072), (24, 8192, 1024), (17, 2080, 8192)])
 def test_swiglu_epilogue_matches_the_two_kernel_chain(m, n, k, per_channel, dtype):
     """One launch (GEMM with SwiGLU epilogue) against GEMM -> 16-bit -> swiglu, on the device and in the oracle.
     The two device paths may sum K in a different order, so a 16-bit projection can differ by one rounding and an
@@ -521,7 +522,7 @@ def test_swiglu_epilogue_limits_and_fallback():
     out = torch.empty(17, 256, dtype=torch.float8_e4m3fn).cuda()
     args = lambda m, n: (a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
                          out_scale.data_ptr(), m, n, 512, 512, _capi.BF16, _capi.EPILOGUE_SWIGLU, None, None)
-    assert lib.hfrk_skinny_gemm_fused(*args(17, 512)) == _capi.BAD_SHAPE      # m > 16: callers run the two kernels
+    assert lib.hfrk_skinny_gemm_fused(*args(17, 512)) == _capi.BAD_SHAPE      # m > 16 on a weight too small to deal out: callers run the two kernels
     assert lib.hfrk_skinny_gemm_fused(*args(8, 496)) == _capi.BAD_SHAPE       # n % 32 != 0
     bad = list(args(8, 512)); bad[3] = out.data_ptr()
     assert lib.hfrk_skinny_gemm_fused(*bad) == _capi.BAD_SHAPE                # base with the SwiGLU epilogue
@@ -545,7 +546,8 @@ def test_swiglu_epilogue_limits_and_fallback():
     assert ((got.cpu().float() - ref.float()).abs() <= tol).all()
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 1024, 2048), (16, 6144, 1024), (3, 2080 * 2, 512), (40, 2080 * 2, 4096), (64, 1024, 2048)])
+@pytest.mark.parametrize("m,n,k", [(8, 1024, 2048), (16, 6144, 1024), (3, 2080 * 2, 512), (40, 2080 * 2, 4096), (64, 1024, 2048),
+                                   (20, 2080 * 2, 1536), (32, 6144, 8192)])
 def test_swiglu_epilogue_under_every_split(m, n, k):
     """Forced plans: grids that cut (gate, up) tile pairs between waves and between workgroups in different places."""
     from hf_rocm_kernels import _capi
@@ -568,9 +570,9 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
             f = out.cpu().float()
             assert not f.isnan().any(), ("k-split", grid)
             assert ((f - ref.float()).abs() <= tol).all(), ("k-split", grid)
-    if m > 16:
+    if m > 32:
         return
-    for grid in sorted({min(g, groups * kc) for g in (256, 200, 64, 7, 1)}):
+    for grid in (sorted({min(g, groups * kc) for g in (256, 200, 64, 7, 1)}) if m <= 16 else []):   # wave-stream plans: up to 16 rows
         plan = _capi.GemmPlan((ma + 3) // 4, 0, 2, ma, grid, groups, kc, 8 * (2 + (ma + 3) // 4) * 4096)
         out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
         st = lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
@@ -583,10 +585,13 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
         assert ((f - ref.float()).abs() <= tol).all(), grid
     if k < 512:
         return
-    # row-split plans: bands of output columns, cut between waves inside a workgroup only
+    # row-split plans: bands of output columns, cut between waves inside a workgroup only (17..32 rows: two activation tiles)
     units = (n // 2 + 3) // 4
+    if m > 16:
+        ma = 6 if m <= 24 else 8
+    rows_lds = 8 * (2 + (ma + 3) // 4) * 4096
     for grid in sorted({min(g, units) for g in (512, 256, 224, 200, 64, 7, 1)}):
-        plan = _capi.GemmPlan(1, -2, 2, ma, grid, units, kc, 8 * 3 * 4096)
+        plan = _capi.GemmPlan(1, -2, 2, ma, grid, units, kc, rows_lds)
         out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
         st = lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
                                         out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
@@ -601,7 +606,7 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
     packed = pack_weight(w.t())
     tiles = (n // 2 + 15) // 16
     for grid in sorted({min(g, tiles) for g in (384, 256, 200, 64, 7, 1)}):
-        plan = _capi.GemmPlan(1, -3, 2, ma, grid, tiles, kc, 8 * 3 * 4096)
+        plan = _capi.GemmPlan(1, -3, 2, ma, grid, tiles, kc, rows_lds)
         outs = []
         for layout in ("row-major", "packed"):
             out = torch.full((m, n // 2), float("nan"), dtype=torch.float32).cuda().to(torch.float8_e4m3fn)
@@ -620,7 +625,7 @@ def test_swiglu_epilogue_under_every_split(m, n, k):
             assert ((f - ref.float()).abs() <= tol).all(), ("rows on tiles", layout, grid)
             outs.append(out.view(torch.uint8))
         assert torch.equal(outs[0], outs[1]), ("rows on tiles: the two layouts differ", grid)
-    one_tile = _capi.GemmPlan(1, -2, 1, ma, 64, units, kc, 8 * 2 * 4096)  # a chunk must hold a gate and an up tile
+    one_tile = _capi.GemmPlan(1, -2, 1, min(ma, 4), 64, units, kc, 8 * 2 * 4096)  # a chunk must hold a gate and an up tile
     assert lib.hfrk_skinny_gemm_fused(a.data_ptr(), w.data_ptr(), out.data_ptr(), None, sa.data_ptr(), 0, sw.data_ptr(), 0,
                                       out_scale.data_ptr(), m, n, k, k, _capi.BF16, _capi.EPILOGUE_SWIGLU,
                                       ctypes.byref(one_tile), torch.cuda.current_stream().cuda_stream) == _capi.INVALID_CONFIG
