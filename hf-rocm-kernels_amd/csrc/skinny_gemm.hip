@@ -951,6 +951,14 @@ static int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed = fa
         if (fits && band_rows >= 48 && k != 2048 && k < 16384 && make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
+    // Packed weights at 17..32 rows: the same kernel on bands of whole tiles, where pairs of tiles deal out evenly over 256
+    // workgroups on a weight of at most 64 MiB.  At 20-24 / 32 rows against the kernels below: 8192 x 8192 13.9 / 14.8 us
+    // against 16.4 / 16.1, 16384 x 4096 13.7 / 14.5 against 17.4 / 17.4, 8192 x 4096 9.0 / 9.4 against 9.5 / 9.5; behind on one
+    // tile per workgroup (4096 x 4096: 7.3 against 6.5), on uneven deals (10240 x 8192: 20.2 against 18.7) and on 8192 x 28672
+    // at 32 rows.
+    if (m <= kRowsMaxM && packed && n % 16 == 0 && (n / 16) % (2 * kNumCU) == 0 && k >= 4096 && (long)n * k <= (64L << 20) &&
+        fill_rows_tiled_plan(m, n, k, 2, kNumCU, plan) == HFRK_SUCCESS)
+        return HFRK_SUCCESS;
     if (k >= 16384 && make_split_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_whole_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_split_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
@@ -1129,6 +1137,17 @@ struct RmsPrologue {
     float epsilon;
     int dtype;
 };
+// The plan of a launch with the RMSNorm prologue: the row-split plan of the shape with one matrix tile per chunk (SwiGLU:
+// the gate and the up tile), whatever the planner or the plan table would take for the plain GEMM.  HFRK_BAD_SHAPE where the
+// prologue does not exist: more than 8 rows, k other than 4096 or 8192 (every thread of a workgroup owns one or two 16-byte
+// pieces of each row), rows that do not deal out over the workgroups.
+static int make_rms_plan(int m, int n, int k, bool swiglu, hfrk_gemm_plan* p) {
+    if (m < 1 || m > kRowsRmsMaxM || (k != 4096 && k != 8192) || n < 1 || (swiglu && n % 32 != 0)) return HFRK_BAD_SHAPE;
+    const int n_eff = swiglu ? n / 2 : n;
+    if (make_rows_plan(m, n_eff, k, p) != HFRK_SUCCESS || p->grid <= m) return HFRK_BAD_SHAPE;
+    return fill_rows_plan(m, n_eff, k, swiglu ? 2 : 1, p->grid, p);
+}
+
 static int gemm_launch(const void* A, const void* B, void* D, const void* base, const float* scale_a, int sa_stride,
                        const float* scale_b, int sb_stride, const float* out_scale, int m, int n, int k, int b_stride,
                        int d_dtype, int epilogue, const hfrk_gemm_plan* user_plan, hipStream_t stream, bool packed = false,
@@ -1188,10 +1207,7 @@ static int gemm_launch(const void* A, const void* B, void* D, const void* base, 
         if (rc != HFRK_SUCCESS) return rc;
         if (rms && (p.wn != -2 || p.wk != (swiglu ? 2 : 1) || p.grid <= m)) return HFRK_INVALID_CONFIG;
     } else if (rms) {
-        // the row-split plan of the shape, one matrix tile per chunk (SwiGLU: the gate and the up tile)
-        const int n_eff = swiglu ? n / 2 : n;
-        if (make_rows_plan(m, n_eff, k, &p) != HFRK_SUCCESS || p.grid <= m) return HFRK_BAD_SHAPE;
-        const int rc = fill_rows_plan(m, n_eff, k, swiglu ? 2 : 1, p.grid, &p);
+        const int rc = make_rms_plan(m, n, k, swiglu, &p);
         if (rc != HFRK_SUCCESS) return rc;
     } else {
         int rc;
@@ -1470,6 +1486,11 @@ int hfrk_skinny_gemm_fused(const void* A, const void* B, void* D, const void* ba
                            int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream) {
     return hfrk::gemm_launch(A, B, D, base, scale_a, sa_stride, scale_b, sb_stride, out_scale, m, n, k, b_stride, d_dtype,
                              epilogue, plan, static_cast<hipStream_t>(stream));
+}
+
+int hfrk_skinny_gemm_rms_plan(int m, int n, int k, int epilogue, hfrk_gemm_plan* plan) {
+    if (!plan || (epilogue != HFRK_EPILOGUE_NONE && epilogue != HFRK_EPILOGUE_SWIGLU)) return HFRK_INVALID_CONFIG;
+    return hfrk::make_rms_plan(m, n, k, epilogue == HFRK_EPILOGUE_SWIGLU, plan);
 }
 
 int hfrk_skinny_gemm_rms_fused(const void* input, const void* residual, void* residual_out, const void* rms_weight,

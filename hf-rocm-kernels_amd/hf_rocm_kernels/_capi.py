@@ -73,6 +73,7 @@ SIGNATURES = {
     "hfrk_skinny_gemm_noalloc": (_i, [_p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_fused": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
     "hfrk_skinny_gemm_rms_fused": (_i, [_p, _p, _p, _p, _f, _p, _i, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, ctypes.POINTER(GemmPlan), _p]),
+    "hfrk_skinny_gemm_rms_plan": (_i, [_i, _i, _i, _i, ctypes.POINTER(GemmPlan)]),
     "hfrk_packed_weight_bytes": (ctypes.c_size_t, [_i, _i]),
     "hfrk_pack_weight": (_i, [_p, _i, _i, _p, _i, _i, _p]),
     "hfrk_unpack_weight": (_i, [_p, _p, _i, _i, _i, _p]),
@@ -123,4 +124,15 @@ def plan(m, n, k):
     """hfrk_skinny_gemm_plan -> GemmPlan (raises on a shape the kernel does not take)."""
     p = GemmPlan()
     check(load().hfrk_skinny_gemm_plan(int(m), int(n), int(k), ctypes.byref(p)), "hfrk_skinny_gemm_plan")
+    return p
+
+
+def rms_plan(m, n, k, epilogue=EPILOGUE_NONE):
+    """hfrk_skinny_gemm_rms_plan -> GemmPlan, or None where the RMSNorm prologue does not exist for the shape
+    (n counts the gate and the up rows together with the SwiGLU epilogue)."""
+    p = GemmPlan()
+    status = load().hfrk_skinny_gemm_rms_plan(int(m), int(n), int(k), int(epilogue), ctypes.byref(p))
+    if status == BAD_SHAPE:
+        return None
+    check(status, "hfrk_skinny_gemm_rms_plan")
     return p

@@ -267,16 +267,16 @@ def skinny_gemm_swiglu(
     return output
 
 
-def rms_prologue_available(m: int, n_rows: int, k: int, b) -> bool:
+def rms_prologue_available(m: int, n_rows: int, k: int, b, swiglu: bool = False) -> bool:
     """Whether `skinny_gemm_rms` runs as one launch: the RMSNorm prologue exists in the row-split kernel -- row-major
-    weights, up to 8 rows, k = 4096 or 8192, and weight rows (output columns with SwiGLU) that deal out evenly over the
-    workgroups, which the library's planner decides (`hfrk_skinny_gemm_plan` returns a row-split plan, wn = -2)."""
-    if isinstance(b, PackedWeight) or m > 8 or k not in (4096, 8192) or torch.compiler.is_compiling():
+    weights, up to 8 rows, k = 4096 or 8192, and weight rows (output columns with SwiGLU: `n_rows` then counts those)
+    that deal out evenly over the workgroups.  The library decides (`hfrk_skinny_gemm_rms_plan`, the function its fused
+    entry point plans with)."""
+    if isinstance(b, PackedWeight) or torch.compiler.is_compiling():
         return False
-    try:
-        return _capi.plan(m, n_rows, k).wn == -2
-    except RuntimeError:
-        return False
+    if swiglu:
+        return _capi.rms_plan(m, 2 * n_rows, k, _capi.EPILOGUE_SWIGLU) is not None
+    return _capi.rms_plan(m, n_rows, k) is not None
 
 
 def skinny_gemm_rms(
@@ -326,7 +326,7 @@ def skinny_gemm_rms(
     if residual_out is None:
         residual_out = torch.empty_like(residual)
     assert residual_out.data_ptr() not in (input.data_ptr(), residual.data_ptr()), "residual_out must not alias input or residual"
-    if not rms_prologue_available(m, n // 2 if swiglu else n, k, b):
+    if not rms_prologue_available(m, n // 2 if swiglu else n, k, b, swiglu):
         return two_launches(residual_out)
     assert scale.numel() == 1 and scale.dtype == torch.float32, "Expected scale to be one float32"
     status = torch.ops._HFRK_C.skinny_gemm_rms_fused(

@@ -225,6 +225,11 @@ int hfrk_skinny_gemm_rms_fused(const void* input, const void* residual, void* re
                                const float* scale_a, const float* scale_b, int sb_stride, const float* out_scale, int m, int n,
                                int k, int b_stride, int d_dtype, int epilogue, const hfrk_gemm_plan* plan, void* stream);
 
+/* Whether hfrk_skinny_gemm_rms_fused has a prologue for a row-major weight of n rows (gate and up rows together with the
+ * SwiGLU epilogue) and, if so, the plan it launches with when none is passed: HFRK_SUCCESS and *plan, or HFRK_BAD_SHAPE.
+ * Host only.  Same decision as the entry point's (one function behind both); the plan table is not consulted. */
+int hfrk_skinny_gemm_rms_plan(int m, int n, int k, int epilogue, hfrk_gemm_plan* plan);
+
 /* Weight load format (no reference counterpart: the reference streams row-major weights through an LDS ring,
  * csrc/op_src/skinny_gemm/producers/n_full_tiles.cu:4-127, and stores fn bits viewed as fnuz,
  * hf_rocm_kernels/utils/fp8.py:27-29).  A weight packed once when the model is loaded is read by the GEMM as one

@@ -6,6 +6,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -296,6 +297,47 @@ def test_plan_rejects_what_the_kernel_cannot_take():
     assert lib.hfrk_skinny_gemm_plan(0, 128, 256, ctypes.byref(p)) == _capi.BAD_SHAPE
     assert lib.hfrk_skinny_gemm_plan(8, 128, 300, ctypes.byref(p)) == _capi.K_NOT_DIVISIBLE_BY_WARPTILE_K
     assert lib.hfrk_skinny_gemm_plan(8, 128, 256, None) == _capi.BAD_SHAPE
+
+
+def test_rms_prologue_predicate_is_the_plan_the_fused_entry_launches_with():
+    """`hfrk_skinny_gemm_rms_plan` is the one decision behind `rms_prologue_available` and `hfrk_skinny_gemm_rms_fused`: a
+    row-split plan (wn = -2) with one weight tile per chunk (two with SwiGLU: gate and up) on more workgroups than rows, or
+    HFRK_BAD_SHAPE -- never another decomposition, whatever the plan table holds for the plain GEMM."""
+    rng = np.random.default_rng(11)
+    lib = _capi.load()
+    seen = {True: 0, False: 0}
+    for _ in range(400):
+        m = int(rng.integers(1, 12))
+        n = int(rng.choice([256, 512, 1000, 2048, 3584, 4096, 4098, 6144, 10240, 14336, 28672])) + 32 * int(rng.integers(0, 3))
+        k = int(rng.choice([2048, 4096, 8192, 4352, 16384]))
+        for epilogue in (_capi.EPILOGUE_NONE, _capi.EPILOGUE_SWIGLU):
+            p = _capi.rms_plan(m, n, k, epilogue)
+            seen[p is not None] += 1
+            if p is None:
+                continue
+            swiglu = epilogue == _capi.EPILOGUE_SWIGLU
+            assert m <= 8 and k in (4096, 8192) and (not swiglu or n % 32 == 0)
+            assert p.wn == -2 and p.wk == (2 if swiglu else 1) and p.grid > m and p.slabs == k // 256
+            n_eff = n // 2 if swiglu else n
+            assert p.panels == (n_eff + 3) // 4
+            _emulate_rows(p)
+    assert seen[True] > 100 and seen[False] > 100
+    assert _capi.rms_plan(9, 4096, 4096) is None and _capi.rms_plan(4, 4096, 2048) is None and _capi.rms_plan(4, 512, 4096) is None
+    assert _capi.rms_plan(4, 4096 + 16, 4096, _capi.EPILOGUE_SWIGLU) is None
+    p = _capi.GemmPlan()
+    assert lib.hfrk_skinny_gemm_rms_plan(4, 4096, 4096, 7, ctypes.byref(p)) == _capi.INVALID_CONFIG
+    assert lib.hfrk_skinny_gemm_rms_plan(4, 4096, 4096, 0, None) == _capi.INVALID_CONFIG
+    # a table entry for the plain GEMM does not change it
+    stream = _capi.GemmPlan(1, 0, 1, 1, 256, 256, 16, 8 * 2 * 4096)
+    before = _capi.rms_plan(4, 4096, 4096)
+    from hf_rocm_kernels import plan_table
+    try:
+        assert lib.hfrk_plan_table_set(4, 4096, 4096, 0, ctypes.byref(stream)) == 0
+        assert plan_table.get_plan(4, 4096, 4096).wn == 0
+        after = _capi.rms_plan(4, 4096, 4096)
+        assert after is not None and (after.wn, after.wk, after.grid) == (before.wn, before.wk, before.grid)
+    finally:
+        plan_table.remove_plan(4, 4096, 4096)
 
 
 def test_plans_for_k_that_ends_inside_a_chunk():

@@ -154,3 +154,38 @@ def test_where_the_prologue_does_not_exist_the_wrapper_runs_two_launches_and_the
                                    _capi.BF16, 0, ctypes.byref(rows_plan), None) == 0
     torch.cuda.synchronize()
     assert torch.equal(out, want)
+
+
+def test_the_predicate_and_the_entry_point_agree_on_random_shapes():
+    """`rms_prologue_available` (hfrk_skinny_gemm_rms_plan) says yes exactly where `hfrk_skinny_gemm_rms_fused` launches, and
+    where it launches the result is the two-launch chain's, bit for bit."""
+    import numpy as np
+    from hf_rocm_kernels import _capi, residual_rms
+    from hf_rocm_kernels.operators.skinny_gemm import rms_prologue_available
+    lib = _capi.load()
+    rng = np.random.default_rng(5)
+    one = torch.ones(1).cuda()
+    seen = {True: 0, False: 0}
+    for case in range(40):
+        m = int(rng.integers(1, 11))
+        n = int(rng.choice([256, 512, 1000, 2048, 3584, 4096, 4098, 6144])) + 4 * int(rng.integers(0, 3))
+        k = int(rng.choice([2048, 4096, 8192]))
+        x, res, w_norm, w8, act_scale, scale = _inputs(m, n, k, torch.bfloat16, seed=100 + case)
+        out = torch.empty(m, n, dtype=torch.bfloat16).cuda()
+        res_out = torch.empty_like(res)
+        st = lib.hfrk_skinny_gemm_rms_fused(x.data_ptr(), res.data_ptr(), res_out.data_ptr(), w_norm.data_ptr(), 1e-5, act_scale.data_ptr(),
+                                            _capi.BF16, w8.data_ptr(), out.data_ptr(), None, scale.data_ptr(), None, 0, None, m, n, k, k,
+                                            _capi.BF16, _capi.EPILOGUE_NONE, None, None)
+        torch.cuda.synchronize()
+        available = rms_prologue_available(m, n, k, w8)
+        seen[available] += 1
+        assert st == (_capi.SUCCESS if available else _capi.BAD_SHAPE), (m, n, k, st, available)
+        if available:
+            normalized, want_res = residual_rms(x, res.clone(), w_norm, 1e-5, scale_tensor=act_scale)
+            want = torch.empty_like(out)
+            plan = _capi.rms_plan(m, n, k)
+            assert lib.hfrk_skinny_gemm_ex(normalized.data_ptr(), w8.data_ptr(), want.data_ptr(), scale.data_ptr(), 0, one.data_ptr(), 0, m, n, k, k,
+                                           _capi.BF16, 0, ctypes.byref(plan), None) == 0
+            torch.cuda.synchronize()
+            assert torch.equal(res_out, want_res) and torch.equal(out, want), (m, n, k)
+    assert seen[True] >= 8 and seen[False] >= 8, seen
