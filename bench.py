@@ -61,8 +61,8 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
 
 HBM_PEAK_GBPS = 8000.0
 # Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0094 x the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55216472}
+# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0096 x the algorithmic bytes.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55226033}
 MEASURED_TRAFFIC_SOURCE = {"llama3-8b": "recorded constant, not measured by this run: profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt "
                                         "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy)"}
 CALIBRATION_COPY_BYTES = 256 << 20
@@ -598,6 +598,8 @@ def run_floor_workload(torch, args):
     lib.probe_empty_launch.argtypes = [ctypes.c_void_p]
     lib.probe_weight_stream.restype = ctypes.c_int
     lib.probe_weight_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    lib.probe_packed_stream.restype = ctypes.c_int
+    lib.probe_packed_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 5 + [ctypes.c_void_p]
 
     def check(status, what):
         if status != 0:
@@ -624,6 +626,13 @@ def run_floor_workload(torch, args):
             check(lib.probe_weight_stream(arena.data_ptr() + offset, sink.data_ptr(), n, k, k, grid, raw()), "probe_weight_stream")
         return call
 
+    def packed_probe(offset, n, k, grid, cyclic):
+        # the same bytes in the packed load format's order: 4 KB chunks, each wave a run of consecutive chunks of its
+        # workgroup's tiles (the GEMM's pattern) or every 8th chunk of them (cyclic)
+        def call():
+            check(lib.probe_packed_stream(arena.data_ptr() + offset, sink.data_ptr(), n, k, grid, 1 if cyclic else 0, 0, raw()), "probe_packed_stream")
+        return call
+
     big_n, big_k = 229376, 8192  # 1.88 GB in one launch
     big = graph_of([probe(0, big_n, big_k)])
     pre_ms = preroll(torch, [big])
@@ -639,10 +648,20 @@ def run_floor_workload(torch, args):
         us, std = time_graph(torch, g, copies, 40)
         hot = graph_of([probe(0, n, k)] * 32)
         us_hot, _ = time_graph(torch, hot, 32, 40)
+        patterns = {}
+        tiles = n // 16
+        for grid in (256, 224, 192):
+            if grid != 256 and tiles % grid != 0:
+                continue
+            for cyclic in (False, True):
+                pg = graph_of([packed_probe(i * wbytes, n, k, grid, cyclic) for i in range(copies)])
+                patterns["%s_%d" % ("cyclic" if cyclic else "runs", grid)] = round(time_graph(torch, pg, copies, 30)[0], 3)
+                del pg
         rows.append({"shape": name, "n": n, "k": k, "weight_mb": round(wbytes / 1e6, 2), "stream_only_us": round(us, 3), "us_std": round(std, 3),
                      "stream_only_gbps": round(wbytes / us / 1e3, 1), "stream_only_frac_of_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
                      "stream_only_us_cache_hot": round(us_hot, 3),
-                     "model_us": round(empty_us + wbytes / sustained / 1e3, 3)})
+                     "model_us": round(empty_us + wbytes / sustained / 1e3, 3),
+                     "packed_stream_only_us": patterns})
         del g, hot
     return {
         "metric": "launch floor and weight-stream-only time of the FP8 skinny GEMM's own load pattern; value = sustained read rate",
@@ -651,7 +670,8 @@ def run_floor_workload(torch, args):
         "dtype": "u8", "data": "synthetic",
         "config": {"workload": "probe kernels of libhfrk_bench_probes.so: probe_empty_launch (256 x 512 threads, 64 KB LDS) x 64 in a graph; "
                                "probe_weight_stream on a %d x %d weight (%.2f GB) and on the eight Llama-3 8B / 70B weights, "
-                               "one graph node per weight copy (HBM-cold) and 32 nodes on one copy (cache-hot)" % (big_n, big_k, big_n * big_k / 1e9),
+                               "one graph node per weight copy (HBM-cold) and 32 nodes on one copy (cache-hot); packed_stream_only_us: probe_packed_stream, "
+                               "the same bytes read as 4 KB chunks in the packed load format's order, <waves take runs of chunks | every 8th chunk>_<workgroups>" % (big_n, big_k, big_n * big_k / 1e9),
                    "preroll_ms": round(pre_ms, 1), "timing": "HIP graph replay, HIP events, median of 40"},
         "roofline": {"bound": "hbm", "achieved": round(sustained, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(sustained / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "hfrk::probe_weight_stream_kernel",
