@@ -11,7 +11,7 @@ void set_last_hip_error(hipError_t e) { g_last_hip_error = static_cast<int>(e); 
 
 extern "C" {
 
-int hfrk_version(void) { return 100; }
+int hfrk_version(void) { return 110; }
 
 int hfrk_last_hip_error(void) { return hfrk::g_last_hip_error; }
 

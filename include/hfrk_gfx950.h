@@ -86,7 +86,8 @@ typedef struct hfrk_gemm_plan {
     int lds_bytes; /* dynamic LDS per workgroup */
 } hfrk_gemm_plan;
 
-/* Library version, for the binding to check. */
+/* Library version, for the binding to check.  110: plan kind wn = -3 (row-split on whole 16-row tiles, both weight layouts),
+ * hfrk_skinny_gemm_rms_plan; the bench-only probe entry points are no longer part of this library (100 had them). */
 int hfrk_version(void);
 
 /* Split-K workspaces.  A GEMM whose row tiles are shared between workgroups parks fp32 partial sums in a workspace
