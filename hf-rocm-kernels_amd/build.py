@@ -25,7 +25,7 @@ OBJ = os.path.join(HERE, "build")
 INCLUDE = os.path.join(ROOT, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["hfrk_common.hip", "skinny_gemm.hip", "skinny_gemm_stream.hip", "skinny_gemm_rows.hip", "skinny_gemm_rows_tiled.hip", "skinny_gemm_ksplit.hip", "residual_rms.hip", "swiglu.hip",
+HIP_SOURCES = ["hfrk_common.hip", "skinny_gemm.hip", "skinny_gemm_plan.hip", "skinny_gemm_stream.hip", "skinny_gemm_rows.hip", "skinny_gemm_rows_tiled.hip", "skinny_gemm_ksplit.hip", "residual_rms.hip", "swiglu.hip",
                "dynamic_quant.hip", "pack_weight.hip", "plan_table_file.hip"]
 PROBE_SOURCE = os.path.join(HERE, "bench_probes", "probe.hip")
 PROBE_LIB = os.path.join(PKG, "benchmarks", "libhfrk_bench_probes.so")

@@ -24,7 +24,7 @@
 //
 // Two things the host decides per launch: where in k a workgroup starts (rotated by its index when all waves of the launch
 // would otherwise read the same offset within 4 KB at every moment, GemmArgs::k_rotate), and how many workgroups there are
-// (the planner in skinny_gemm.hip: whole 16-row tiles where a grid of 224..256 gives them, twice the workgroups for short
+// (the planner in skinny_gemm_plan.hip: whole 16-row tiles where a grid of 224..256 gives them, twice the workgroups for short
 // bands at up to 4 rows, no bands of exactly 512 KB).
 //
 // Replaces, for these shapes, the reference's csrc/op_src/skinny_gemm/skinny_gemm_kernel.cu:6-79 with its producers and

@@ -19,22 +19,31 @@ def _oracle():
     return og
 
 
-def check_against_oracle(out, a, b, sa, sb, base=None, rtol=1e-2, atol=1e-2):
+def oracle_checker(a, b, sa, sb, out_dtype, base=None, rtol=1e-2, atol=1e-2):
+    """The oracle's answers for one set of inputs, computed once: returns check(out) for any number of device results of
+    the same product (e.g. one per plan)."""
     og = _oracle()
     a_c, b_c = a.cpu(), b.cpu()
     sa_c, sb_c = sa.cpu(), sb.cpu()
     base_c = None if base is None else base.cpu()
-    ref32 = og.reference_skinny_gemm(a_c, b_c, sa_c, sb_c, output=base_c, out_dtype=out.dtype)
+    ref32 = og.reference_skinny_gemm(a_c, b_c, sa_c, sb_c, output=base_c, out_dtype=out_dtype).float()
     exact = og.exact_skinny_gemm(a_c, b_c, sa_c, sb_c, output=base_c)
-    got = out.cpu()
-    assert not got.isnan().any()
-    err32 = (got.float() - ref32.float()).abs()
-    tol = atol + rtol * ref32.float().abs()
-    assert (err32 <= tol).all(), f"max excess over rtol/atol: {(err32 - tol).max().item()}"
-    err_exact = (got.double() - exact).abs()
-    bound = og.error_bound(a_c, b_c, sa_c, sb_c, out.dtype, exact)
-    worst = (err_exact / bound).max().item()
-    assert worst <= 1.0, f"error is {worst} x the bound (1 ulp + 2^-16 sum|a b|) from the exact product"
+    tol = atol + rtol * ref32.abs()
+    bound = og.error_bound(a_c, b_c, sa_c, sb_c, out_dtype, exact)
+
+    def check(out):
+        assert out.dtype == out_dtype
+        got = out.cpu()
+        assert not got.isnan().any()
+        err32 = (got.float() - ref32).abs()
+        assert (err32 <= tol).all(), f"max excess over rtol/atol: {(err32 - tol).max().item()}"
+        worst = ((got.double() - exact).abs() / bound).max().item()
+        assert worst <= 1.0, f"error is {worst} x the bound (1 ulp + 2^-16 sum|a b|) from the exact product"
+    return check
+
+
+def check_against_oracle(out, a, b, sa, sb, base=None, rtol=1e-2, atol=1e-2):
+    oracle_checker(a, b, sa, sb, out.dtype, base=base, rtol=rtol, atol=atol)(out)
 
 
 def run_ex(a, b, sa, sb, out, accumulate, plan=None):
@@ -172,11 +181,12 @@ def test_every_plan_gives_the_same_answer(m, n, k):
     a, b, sa, sw = generate_llama_gemm_data(m, n, k, seed=7)
     plans = all_plans(m, n, k)
     assert plans
+    check = oracle_checker(a, b, sa, sw, torch.bfloat16)
     for p in plans:
         out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         run_ex(a, b, sa, sw, out, accumulate=False, plan=p)
         try:
-            check_against_oracle(out, a, b, sa, sw)
+            check(out)
         except AssertionError as e:
             raise AssertionError(f"plan {p.as_dict()}: {e}")
 
