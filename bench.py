@@ -60,11 +60,15 @@ for _p in (ROOT, os.path.join(ROOT, "hf-rocm-kernels_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
-# Mean HBM bytes per GEMM launch of a llama3-8b step (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised in profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt: 1.0096 x the algorithmic bytes.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 55226033}
-MEASURED_TRAFFIC_SOURCE = {"llama3-8b": "recorded constant, not measured by this run: profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt "
-                                        "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy)"}
+# Mean HBM bytes per GEMM launch of a step (fetched + written), from FETCH_SIZE / WRITE_SIZE counter runs of this script
+# summarised under profiles/: 1.009-1.010 x the algorithmic bytes.  Keys: (workload, packed weights).
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("llama3-8b", False): 55226033, ("llama3-8b", True): 55230061, ("llama3-70b", False): 216609072}
+_TRAFFIC_HOW = " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 256 MiB copy)"
+MEASURED_TRAFFIC_SOURCE = {
+    ("llama3-8b", False): "recorded constant, not measured by this run: profiles/skinny_gemm_llama3_8b_decode_hbm_traffic.txt" + _TRAFFIC_HOW,
+    ("llama3-8b", True): "recorded constant, not measured by this run: profiles/skinny_gemm_llama3_70b_and_packed_8b_hbm_traffic.txt" + _TRAFFIC_HOW,
+    ("llama3-70b", False): "recorded constant, not measured by this run: profiles/skinny_gemm_llama3_70b_and_packed_8b_hbm_traffic.txt" + _TRAFFIC_HOW,
+}
 CALIBRATION_COPY_BYTES = 256 << 20
 
 WORKLOADS = {
@@ -793,8 +797,8 @@ def main():
                    "us_per_call_mean": round(ms_per_step * 1e3 / calls, 3), "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": None if args.packed else MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
-                     "traffic_source": None if args.packed else MEASURED_TRAFFIC_SOURCE.get(args.workload),
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, bool(args.packed))) if args.ms is None else None,
+                     "traffic_source": MEASURED_TRAFFIC_SOURCE.get((args.workload, bool(args.packed))) if args.ms is None else None,
                      "kernel": kernel,
                      "bytes_per_launch": round(step_bytes / calls), "us_per_launch": round(ms_per_step * 1e3 / calls, 3)},
     }
