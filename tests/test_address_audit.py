@@ -505,3 +505,54 @@ def test_library_refuses_grids_no_test_covers():
     assert "small-weights" not in inspect.getsource(grid_search)
     for p in grid_search.candidate_plans(m, 4096, k, [192, 512, 1024]):
         assert p.grid <= (512 if p.wn in (0, -2, -3) else 256)
+
+
+def test_whatever_the_plan_check_accepts_stays_inside_its_buffers():
+    """Seeded random plans of every kind on random small shapes, offered to the library the way a plan table or a caller would
+    (hfrk_plan_table_set runs the launcher's check): every plan it accepts is audited, in the weight layout it was accepted
+    for.  The point is the converse of the hand-made cases above -- not "these plans are fine" but "the check lets nothing
+    through that is not"."""
+    import random
+    rng = random.Random(20250)
+    lib = _capi.load()
+    accepted = {-3: 0, -2: 0, -1: 0, 0: 0, 1: 0}
+    offered = 0
+    while min(accepted.values()) < 40 and offered < 60000:
+        m = rng.choice([1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 25, 32, 33, 48, 64])
+        n = rng.choice([16 * rng.randrange(1, 160), 4 * rng.randrange(1, 640), rng.randrange(1, 2600)])
+        k = 256 * rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 32]) if rng.random() < 0.9 else 16 * rng.randrange(1, 200)
+        packed = rng.random() < 0.4
+        kind = rng.choice([-3, -2, -1, 0, 1])
+        mt = (m + 15) // 16
+        ma = (m + 3) // 4 if m <= 16 else rng.choice([6, 8])
+        grid = rng.choice([1, 2, 7, 8, 64, 100, 192, 200, 256, 264, 320, 512, 513, 1024])
+        if kind in (-3, -2):
+            rt = rng.choice([1, 2])
+            panels = -(-n // 16) if kind == -3 else -(-n // 4)
+            p = _capi.GemmPlan(1, kind, rt, rng.choice([ma, ma, ma + 1, 4]), min(grid, panels) if rng.random() < 0.9 else grid, panels,
+                               k // 256, 8 * (rt + (max(ma, 1) + 3) // 4) * 4096)
+        elif kind == -1:
+            wave_k = rng.choice([256, 512, 1024])
+            tiles, windows = -(-n // 16), max(1, k // (8 * wave_k))
+            p = _capi.GemmPlan(mt, -1, wave_k // 256, 0, min(grid, tiles * windows), tiles, windows, 8 * (wave_k // 256) * 4096 + 16 * mt * 1024)
+        elif kind == 0:
+            rt = rng.choice([1, 2])
+            groups, kc = -(-n // (16 * rt)), -(-k // 256)
+            p = _capi.GemmPlan((ma + 3) // 4, 0, rt, ma, min(grid, groups * kc), groups, kc, 8 * (rt + (ma + 3) // 4) * 4096)
+        else:
+            wn, ch, rt = rng.choice([1, 2, 4, 8]), rng.choice([1, 2]), rng.choice([1, 1, 2])
+            wk = 8 // wn
+            ks = 256 * wk * ch
+            panels, slabs = -(-n // (16 * wn * rt)), max(1, k // ks)
+            p = _capi.GemmPlan(mt, wn * rt, wk, ch, min(grid, panels * slabs), panels, slabs, 8 * rt * 4096 + 2 * 16 * mt * ks)
+        offered += 1
+        status = lib.hfrk_plan_table_set(m, n, k, int(packed), ctypes.byref(p))
+        if status != _capi.SUCCESS:
+            continue
+        lib.hfrk_plan_table_set(m, n, k, int(packed), None)   # (take it out again)
+        if accepted[min(p.wn, 1)] >= 60:
+            continue
+        accepted[min(p.wn, 1)] += 1
+        assert p.grid <= (512 if p.wn in (-3, -2, 0) else 256)
+        assert audit(m, n, k, p, packed=packed) > 0, (m, n, k, packed, p.as_dict())
+    assert min(accepted.values()) >= 40, (accepted, offered)
