@@ -91,7 +91,7 @@ constexpr int rows_rms_lds_bytes(int act_loads, int row_tiles, int k) {
 // the same kernel on bands of whole 16-row tiles (skinny_gemm_rows_tiled.hip): args.rows_q / rows_r count 16-row tiles (with swiglu:
 // tiles of 16 output columns), args.packed selects the packed load format; no RMSNorm prologue
 int launch_rows_tiled_kernel(const GemmArgs& args, int act_loads, int row_tiles, bool swiglu, int lds_bytes, hipStream_t stream);
-constexpr int kRowsMaxM = 32;  // 17..32 rows: act_loads 6 (up to 24 rows) or 8, two matrix tiles per chunk, plain epilogue
+constexpr int kRowsMaxM = 32;  // 17..32 rows: act_loads 6 (up to 24 rows) or 8, two matrix tiles per chunk
 constexpr int rows_act_loads(int m) { return m <= 16 ? (m + 3) / 4 : m <= 24 ? 6 : 8; }
 constexpr int rows_lds_bytes(int row_tiles, int act_loads) { return kGemmWaves * (row_tiles + (act_loads + 3) / 4) * kTileBytes; }
 constexpr bool rows_variant_exists(int act_loads, int row_tiles) {

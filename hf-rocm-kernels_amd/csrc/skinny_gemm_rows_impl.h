@@ -69,7 +69,7 @@ __global__ void __launch_bounds__(kGemmThreads) skinny_gemm_rows_kernel(const Ge
     constexpr int PT = SWIGLU ? 4 : 4 * RT;  // 4-row units a chunk can hold (SwiGLU: 16 output columns, their gate and their up rows)
     static_assert(!SWIGLU || RT == 2, "the SwiGLU epilogue pairs one gate tile with one up tile");
     static_assert(!RMS || MA <= 2, "the RMSNorm prologue keeps every row in registers: up to 8 rows");
-    constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles: 2 from 17 rows on (plain epilogue, two matrix tiles per chunk)
+    constexpr int MT = (MA + 3) / 4;  // 16-row activation tiles: 2 from 17 rows on (two matrix tiles per chunk, either epilogue)
     static_assert(MT == 1 || (MT == 2 && RT == 2 && !RMS), "above 16 rows: two weight tiles per chunk, no RMSNorm prologue");
     constexpr uint32_t kOutOfRange = 0x80000000u;
     constexpr int kWaveLds = (RMS ? RT : RT + MT) * kTileBytes;  // RT weight tiles, MT activation tiles (RMS: rows staged once instead)
