@@ -155,10 +155,14 @@ int fill_rows_tiled_plan(int m, int n, int k, int row_tiles, int grid_hint, hfrk
 //    against 39.4 at 8 rows);
 //  * not on the largest weights (57344 x 8192: 73.6-76.5 us against 72.8 for the workgroup kernel and 68.5 for the row-major
 //    weight -- a run of 56 contiguous chunks per wave is the slowest way to read that much memory).
+//  * from 144 tiles (2304 rows, the smallest weight measured) on, one tile per workgroup: 2304..3040 rows x k = 2048..14336 at 1 /
+//    8 / 16 rows are 4-49 % faster than the wave-stream split and, at k = 2048, 0-37 % faster than the K-split kernel (2304 x
+//    4096: 4.3 / 4.6 / 5.0 us against 6.3 / 6.5 / 6.7; 3040 x 2048: 3.6 / 4.0 / 4.2 against 4.9 / 5.0 / 5.0; 2304 x 14336 at 16 rows,
+//    10.9 against 10.3, is the one case behind), so the rule comes before the K-split rule for small weights.
 int make_rows_tiled_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     if (m > 16 || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
     const long tiles = (n + 15) / 16;
-    if (tiles < 3 * kNumCU / 4 || (long)n * k > (256L << 20)) return HFRK_INVALID_CONFIG;
+    if (tiles < 9 * kNumCU / 16 || (long)n * k > (256L << 20)) return HFRK_INVALID_CONFIG;
     const long busiest = (tiles + kNumCU - 1) / kNumCU;
     long grid = (tiles + busiest - 1) / busiest;
     grid = (grid + 7) / 8 * 8;
@@ -169,6 +173,26 @@ int make_rows_tiled_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
     const long band_tiles = (tiles + grid - 1) / grid;
     const int row_tiles = (band_tiles >= 2 && (m >= 9 || k > 16384)) ? 2 : 1;
     return fill_rows_tiled_plan(m, n, k, row_tiles, (int)grid, plan);
+}
+
+// Packed weights at 17..32 rows (two activation tiles, two weight tiles per chunk): the grid.  One tile each while there are
+// at most 256 tiles; one pair of tiles each from 160 pairs on (5120 rows on 160 workgroups, 6144 on 192); more pairs only
+// where they deal out evenly over 192..256 workgroups (13312 rows: 2 pairs each on 208).  Uneven deals of more than 256
+// pairs are left to the other kernels (10240 rows, 320 pairs: 3-9 % behind them on 192 workgroups at k = 3072, 5120, 14336).
+static int make_rows_tiled_pairs_plan(int m, int n, int k, hfrk_gemm_plan* plan) {
+    if (m <= 16 || m > kRowsMaxM || k < 512 || k % 256 != 0) return HFRK_INVALID_CONFIG;
+    const long tiles = (n + 15) / 16, pairs = (tiles + 1) / 2;
+    long grid = 0;
+    if (tiles <= kNumCU) {
+        grid = tiles;
+    } else if (pairs <= kNumCU) {
+        grid = pairs >= 5 * kNumCU / 8 ? pairs : kNumCU;
+    } else {
+        for (long g = kNumCU; g >= 3 * kNumCU / 4 && !grid; g -= 8)
+            if (tiles % 2 == 0 && pairs % g == 0) grid = g;
+        if (!grid) return HFRK_INVALID_CONFIG;
+    }
+    return fill_rows_tiled_plan(m, n, k, 2, (int)grid, plan);
 }
 
 // 17 <= m <= 64 (valid from 1): the waves of a workgroup split K windows of 8*wave_k bytes, activations in registers
@@ -284,6 +308,9 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool
         // 6144 x 3072 on 192 workgroups 9.2 / 9.6 against 10.6 / 10.9, 5120 x 5120 on 160 11.8 / 12.4 against 12.9 / 13.1; at
         // 64 rows level or 9 % behind, at k = 8192 18-27 % behind, at k = 2048 / 4096 7-24 % behind the K-split kernel)
         if (h == 32 && (panels > kNumCU || k > 5120 || k == 2048 || k == 4096 || m > 48)) continue;
+        // (a packed 128-row panel at k = 8192 is 1 MB of contiguous bytes per workgroup: 28672 x 8192 at 20 / 32 rows 48.9 / 48.0 us
+        // against 41.0 / 41.8 on 64-row panels, two per workgroup; 24576 x 8192 42.0 against 36.4 for the rules below)
+        if (h == 128 && packed && k == 8192) continue;
         long g_try[2] = {0, 0};  // several panels each on 224..256 workgroups; one panel each on fewer
         if (k <= 8192)
             for (long g = kNumCU; g >= 7 * kNumCU / 8 && !g_try[0]; g -= 8)
@@ -296,9 +323,6 @@ static int make_whole_panel_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool
             if (h == 64) one_each = panels >= (k <= 5120 ? 160 : k <= 8192 ? 192 : 208) && k <= 14336 && !(k == 4096 && m > 32 && panels < 208);
             if (h == 64 && k == 16384 && m <= 48) one_each = panels >= 208;
             if (h == 128) one_each = panels >= 192 || (panels >= 160 && k <= 8192 && k != 4096 && k != 2048);
-            // (packed weights, 24576 x 8192: 42.0 / 41.9 / 45.2 us at 20 / 32 / 64 rows against 36.4 / 36.6 / 43.2 for the rules
-            // below -- a panel is 1 MB of contiguous bytes there; k = 3072, 5120 and 16384 gain 11-24 % in both layouts)
-            if (h == 128 && packed && k == 8192) one_each = false;
             if (h == 32) one_each = panels >= 160;
             if (one_each) g_try[1] = panels;
         }
@@ -361,11 +385,11 @@ int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed) {
         // tile through the workspace; one workgroup per tile, its 8 waves splitting K, finishes inside the workgroup
         // (2048 x 2048: 3.8 against 5.2 us; 2048 x 4096: 5.0 against 5.8).
         const long chunks = (long)((n + 15) / 16) * (k / 256);
+        if (packed && make_rows_tiled_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // bands of whole 16-row tiles
         if (chunks <= (long)kNumCU * kGemmWaves && make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         // Bands of rows per workgroup: nothing crosses workgroups and the end of the launch is short (0.3-1.3 us less than
         // the wave-stream split on every Llama-3 8B / 70B projection at 1..16 rows).
         if (!packed && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // (bands of any multiple of 4 rows: row-major weights only)
-        if (packed && make_rows_tiled_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // bands of whole 16-row tiles
         return make_stream_plan(m, n, k, plan);
     }
     // 17..32 rows in the row-split kernel (two activation tiles): every workgroup then pulls all m x k activation bytes out
@@ -380,7 +404,18 @@ int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed) {
     // 7.3 / 7.35 against 8.5, 4096 x 5120 8.4 / 8.5 / 9.2 / 9.35 against 9.8-9.9, 5120 x 8192 11.0 / 11.3 / 12.1 / 12.4 against
     // 13.7-13.8.  Not where one K-split window covers k and its tiles deal out evenly (3072 and 4096 rows at k = 2048 and
     // 4096: level or 0.3-0.9 us behind), nor above 24 rows at k = 8192 on bands under 20 rows or at k = 2048.
-    if (m <= kRowsMaxM && !packed) {
+    // Packed weights first take the kernel where pairs of tiles deal out evenly over 256 workgroups on a weight of at most 64 MiB
+    // (at 20-24 / 32 rows: 8192 x 8192 13.9 / 14.8 us against 16.4 / 16.1 for the kernels below, 16384 x 4096 13.7 / 14.5 against
+    // 17.4 / 17.4, 8192 x 4096 9.0 / 9.4 against 9.5 / 9.5), and otherwise follow the same rule on bands of whole tiles
+    // (make_rows_tiled_pairs_plan).  A sweep of 11 row counts x 5 k at 20 and 32 rows: where the rule takes the kernel the
+    // packed weight gains 2-35 % over the kernels below (3072 x 3072 6.3 / 6.8 us against 8.5, 4096 x 5120 8.1 / 8.9 against 9.7,
+    // 5120 x 8192 11.5 / 12.9 against 14.0, 6144 x 8192 11.9 against 13.5 at 20 rows, 13312 x 4096 12.2 against 13.9) or is level;
+    // where it does not, the kernel is 3-14 % behind.  On a packed weight whole 64-row
+    // panels do not come first at k = 4096 (13312 / 14336 x 4096 at 20 rows: 12.1 / 12.5 us against 13.9 / 14.4).
+    if (m <= kRowsMaxM && packed && n % 16 == 0 && (n / 16) % (2 * kNumCU) == 0 && k >= 4096 && (long)n * k <= (64L << 20) &&
+        fill_rows_tiled_plan(m, n, k, 2, kNumCU, plan) == HFRK_SUCCESS)
+        return HFRK_SUCCESS;
+    if (m <= kRowsMaxM) {
         const long band_rows = 4 * (((long)(n + 3) / 4 + kNumCU - 1) / kNumCU);
         // (k = 2048 above 24 rows: the K-split kernel is 3-4 % ahead, 6144 x 2048 6.5 against 6.7 us)
         bool fits = band_rows >= 24 && (m <= 24 ? (band_rows <= 64 && k <= 16384) : (band_rows <= 32 && k >= 3072 && k <= 8192));
@@ -389,17 +424,11 @@ int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed) {
         // From 12288 weight rows on, whole 64-row panels per workgroup come first where they exist: at 20 / 24 rows 12288 x
         // 8192 19.8 / 20.0 us against 20.5 / 21.2, 13312 x 8192 20.6 / 20.8 against 21.7 / 22.2, 14336 x 5120 15.7 / 15.8 against
         // 17.2 / 17.7, 16384 x 14336 39.4 / 39.2 against 42.1 / 43.3; level at k = 4096 and 16384 and on 10240 rows.
-        if (fits && band_rows >= 48 && k != 2048 && k < 16384 && make_whole_panel_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
-        if (fits && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
+        if (fits && band_rows >= 48 && k != 2048 && k < 16384 && !(packed && k == 4096) &&
+            make_whole_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS)
+            return HFRK_SUCCESS;
+        if (fits && (packed ? make_rows_tiled_pairs_plan(m, n, k, plan) : make_rows_plan(m, n, k, plan)) == HFRK_SUCCESS) return HFRK_SUCCESS;
     }
-    // Packed weights at 17..32 rows: the same kernel on bands of whole tiles, where pairs of tiles deal out evenly over 256
-    // workgroups on a weight of at most 64 MiB.  At 20-24 / 32 rows against the kernels below: 8192 x 8192 13.9 / 14.8 us
-    // against 16.4 / 16.1, 16384 x 4096 13.7 / 14.5 against 17.4 / 17.4, 8192 x 4096 9.0 / 9.4 against 9.5 / 9.5; behind on one
-    // tile per workgroup (4096 x 4096: 7.3 against 6.5), on uneven deals (10240 x 8192: 20.2 against 18.7) and on 8192 x 28672
-    // at 32 rows.
-    if (m <= kRowsMaxM && packed && n % 16 == 0 && (n / 16) % (2 * kNumCU) == 0 && k >= 4096 && (long)n * k <= (64L << 20) &&
-        fill_rows_tiled_plan(m, n, k, 2, kNumCU, plan) == HFRK_SUCCESS)
-        return HFRK_SUCCESS;
     if (k >= 16384 && make_split_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_whole_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
     if (make_split_panel_plan(m, n, k, plan, packed) == HFRK_SUCCESS) return HFRK_SUCCESS;
