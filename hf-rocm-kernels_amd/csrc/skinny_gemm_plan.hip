@@ -386,6 +386,9 @@ int make_plan(int m, int n, int k, hfrk_gemm_plan* plan, bool packed) {
         // (2048 x 2048: 3.8 against 5.2 us; 2048 x 4096: 5.0 against 5.8).
         const long chunks = (long)((n + 15) / 16) * (k / 256);
         if (packed && make_rows_tiled_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;  // bands of whole 16-row tiles
+        // (from 2304 rows on, the smallest weight measured against it, the row-split kernel is ahead of that rule as well: 2304..4096
+        // x 2048 at 1 / 8 / 16 rows 3.4-3.95 / 3.7-4.2 / 3.9-4.3 us against 3.8-4.3 / 4.0-4.5 / 4.1-4.6)
+        if (!packed && n >= 2304 && make_rows_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         if (chunks <= (long)kNumCU * kGemmWaves && make_ksplit_plan(m, n, k, plan) == HFRK_SUCCESS) return HFRK_SUCCESS;
         // Bands of rows per workgroup: nothing crosses workgroups and the end of the launch is short (0.3-1.3 us less than
         // the wave-stream split on every Llama-3 8B / 70B projection at 1..16 rows).
